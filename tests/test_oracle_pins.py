@@ -1,0 +1,203 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.  CPU only.
+
+* quantizer: golden vectors written from the reference kernel under Triton's CPU
+  interpreter (tests/golden/quant_golden.npz), hand-worked ties, invariants;
+* attention: reduction to torch's SDPA (scale = ln 2) on the dequantized operands,
+  uniform-V / single-tile / fully-masked closed forms, numpy-vs-C agreement;
+* K mean: agreement with the fp32 mean to one 16-bit ulp and an exact case.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from golden_io import load_cases
+from oracle import c_oracle as C
+from oracle import sage_oracle as O
+
+CASES = load_cases()
+
+
+def _same_scale(a, b):
+    return torch.equal(a, b)
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["name"] for c in CASES])
+@pytest.mark.parametrize("impl", ["numpy", "c"])
+def test_quantizer_matches_reference_golden(case, impl):
+    fn = O.per_block_int8 if impl == "numpy" else C.per_block_int8
+    q8, qs, k8, ks = fn(case["q"], case["k"], km=case["km"], **case["kw"])
+    assert q8.dtype == torch.int8 and k8.dtype == torch.int8
+    assert qs.dtype == torch.float32 and ks.dtype == torch.float32
+    assert q8.shape == case["q_int8"].shape and qs.shape == case["q_scale"].shape
+    assert torch.equal(q8, case["q_int8"])
+    assert torch.equal(k8, case["k_int8"])
+    assert _same_scale(qs, case["q_scale"])
+    assert _same_scale(ks, case["k_scale"])
+
+
+def test_quantizer_hand_worked_ties():
+    # K path multiplies by nothing; amax = 127 -> scale = 1, so y = x exactly.
+    k = torch.zeros(1, 1, 64, 64, dtype=torch.float32)
+    xs = [127.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49999997, -0.49999997, 0.4999999, 126.5, -126.5, 126.49999]
+    want = [127, 1, -1, 2, -2, 3, -3, 1, -1, 0, 127, -127, 126]  # half away from zero; 0.49999997+0.5 rounds up to 1.0f
+    k[0, 0, 0, : len(xs)] = torch.tensor(xs)
+    q = torch.ones(1, 1, 128, 64)
+    for fn in (O.per_block_int8, C.per_block_int8):
+        _, _, k8, ks = fn(q, k)
+        assert ks.item() == 1.0
+        assert k8[0, 0, 0, : len(xs)].tolist() == want
+
+
+def test_quantizer_q_scale_constant():
+    # sm_scale * 1.44269504 is a python double packed to fp32: D=128 -> 0x3e0293ee, D=64 -> 0x3e38aa3b
+    assert np.float32(128 ** -0.5 * 1.44269504).view(np.uint32) == 0x3E0293EE
+    assert np.float32(64 ** -0.5 * 1.44269504).view(np.uint32) == 0x3E38AA3B
+    q = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16)
+    q[0, 0, 5, 7] = 2.0
+    _, qs, _, _ = O.per_block_int8(q, q)
+    assert qs.item() == float(np.float32(2.0) * np.float32(128 ** -0.5 * 1.44269504) / np.float32(127.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_quantizer_invariants(dtype):
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(2, 3, 300, 64, generator=g).to(dtype)
+    k = (torch.randn(2, 3, 200, 64, generator=g) * 3).to(dtype)
+    q8, qs, k8, ks = O.per_block_int8(q, k)
+    c8, cs, ck8, cks = C.per_block_int8(q, k)
+    assert torch.equal(q8, c8) and torch.equal(k8, ck8) and torch.equal(qs, cs) and torch.equal(ks, cks)
+    for x8, s, x, blk, mul in ((q8, qs, q, 128, np.float32(64 ** -0.5 * 1.44269504)), (k8, ks, k, 64, np.float32(1.0))):
+        assert int(x8.min()) >= -127  # symmetric: -128 never appears
+        xf = torch.from_numpy(x.float().numpy() * mul)
+        nb = s.shape[-1]
+        for ib in range(nb):
+            blk_x = xf[:, :, ib * blk:(ib + 1) * blk]
+            blk_8 = x8[:, :, ib * blk:(ib + 1) * blk]
+            amax = blk_x.abs().amax(dim=(-1, -2))
+            assert torch.equal(s[..., ib], amax / torch.tensor(127.0))
+            assert torch.equal(blk_8.abs().amax(dim=(-1, -2)), torch.full_like(amax, 127).to(torch.int8))
+            err = (blk_8.float() * s[..., ib, None, None] - blk_x).abs()
+            assert bool((err <= s[..., ib, None, None] * 0.5 * (1 + 1e-5)).all())
+
+
+def test_c_half_conversions_match_torch():
+    lib = C.lib()
+    allh = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    f = allh.float()
+    for i in range(0, 65536, 7):
+        v = f[i].item()
+        if math.isnan(v):
+            continue
+        assert lib.sage_oracle_f16_to_f32(i) == v
+        assert lib.sage_oracle_f32_to_f16(v) == i
+    g = torch.Generator().manual_seed(11)
+    x = torch.cat([torch.randn(4000, generator=g) * s for s in (1e-7, 1e-4, 1.0, 300.0, 7e4)])
+    h = x.to(torch.float16).view(torch.int16).to(torch.int32) & 0xFFFF
+    b = x.to(torch.bfloat16).view(torch.int16).to(torch.int32) & 0xFFFF
+    for xi, hi, bi in zip(x.tolist(), h.tolist(), b.tolist()):
+        assert lib.sage_oracle_f32_to_f16(xi) == hi
+        assert lib.sage_oracle_f32_to_bf16(xi) == bi
+
+
+def _rand_quantized(g, b, hq, hkv, m, n, d, vdtype=torch.float16):
+    q = torch.randn(b, hq, m, d, generator=g).to(vdtype)
+    k = torch.randn(b, hkv, n, d, generator=g).to(vdtype)
+    v = torch.randn(b, hkv, n, d, generator=g).to(vdtype)
+    return (*O.per_block_int8(q, k), v)
+
+
+def test_attention_dequant_reduces_to_sdpa():
+    g = torch.Generator().manual_seed(2026)
+    q8, qs, k8, ks, v = _rand_quantized(g, 1, 4, 2, 200, 150, 64)
+    out, lse = O.attention_dequant(q8, k8, v, qs, ks)
+    qd = q8.float() * qs.repeat_interleave(128, -1)[..., :200, None]
+    kd = k8.float() * ks.repeat_interleave(64, -1)[..., :150, None]
+    ref = F.scaled_dot_product_attention(qd, kd.repeat_interleave(2, 1), v.float().repeat_interleave(2, 1),
+                                         scale=math.log(2.0))
+    torch.testing.assert_close(out, ref, atol=2e-5, rtol=1e-4)
+    s2 = qd @ kd.repeat_interleave(2, 1).transpose(-1, -2)
+    torch.testing.assert_close(lse, torch.log2(torch.exp2(s2.double()).sum(-1)).float(), atol=1e-4, rtol=1e-5)
+
+
+def test_attention_closed_forms():
+    g = torch.Generator().manual_seed(5)
+    q8, qs, k8, ks, v = _rand_quantized(g, 1, 2, 2, 130, 200, 64)
+    # uniform V rows -> every output row equals that row, whatever the weights
+    vu = v[:, :, :1].expand_as(v).contiguous()
+    for fn in (O.attention_dequant, O.attention_blockwise, C.attention_blockwise):
+        out, _ = fn(q8, k8, vu, qs, ks)
+        torch.testing.assert_close(out, vu[:, :, :1].float().expand_as(out), atol=2e-3, rtol=2e-3)
+    # all-False bool mask: every tile is skipped -> o = 0, lse = -inf (kernel semantics only)
+    mask = torch.zeros(1, 2, 130, 200, dtype=torch.bool)
+    for fn in (O.attention_blockwise, C.attention_blockwise):
+        out, lse = fn(q8, k8, v, qs, ks, attn_mask=mask)
+        assert float(out.abs().max()) == 0.0 and bool(torch.isinf(lse).all()) and bool((lse < 0).all())
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("mask_kind", [None, "bool", "additive", "causal"])
+def test_blockwise_agrees_with_dequant(layout, mask_kind):
+    g = torch.Generator().manual_seed(7)
+    b, hq, hkv, m, n, d = 1, 2, 1, 129, 257, 64
+    q8, qs, k8, ks, v = _rand_quantized(g, b, hq, hkv, m, n, d)
+    if layout == "NHD":
+        q8, k8, v = (t.transpose(1, 2).contiguous() for t in (q8, k8, v))
+    mask, causal = None, False
+    if mask_kind == "bool":
+        mask = torch.ones(b, hq, m, n, dtype=torch.bool)
+        mask[..., ::3] = False
+    elif mask_kind == "additive":
+        mask = torch.zeros(b, hq, m, n)
+        mask[..., ::3] = -2.0
+    elif mask_kind == "causal":
+        causal = True
+    ref, ref_lse = O.attention_dequant(q8, k8, v, qs, ks, layout, attn_mask=mask, causal=causal)
+    for fn in (O.attention_blockwise, C.attention_blockwise):
+        out, lse = fn(q8, k8, v, qs, ks, layout, attn_mask=mask, causal=causal)
+        torch.testing.assert_close(out, ref, atol=3e-3, rtol=3e-3)  # P rounded to fp16 before PV
+        torch.testing.assert_close(lse, ref_lse, atol=1e-4, rtol=1e-5)
+    a, _ = O.attention_blockwise(q8, k8, v, qs, ks, layout, attn_mask=mask, causal=causal)
+    c, _ = C.attention_blockwise(q8, k8, v, qs, ks, layout, attn_mask=mask, causal=causal)
+    torch.testing.assert_close(a, c, atol=1e-5, rtol=1e-5)
+
+
+def test_causal_mask_convention():
+    cm = O.causal_mask(3, 5)[0, 0]
+    assert cm.tolist() == [[True, True, True, False, False], [True, True, True, True, False], [True] * 5]
+    assert torch.equal(O.causal_mask(4, 4)[0, 0], torch.ones(4, 4).tril().bool())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+def test_k_mean_fixed_order(dtype, layout):
+    g = torch.Generator().manual_seed(9)
+    k = (torch.randn(2, 3, 333, 64, generator=g) + torch.randn(1, 3, 1, 64, generator=g) * 2).to(dtype)
+    if layout == "NHD":
+        k = k.transpose(1, 2).contiguous()
+    seq = 2 if layout == "HND" else 1
+    a = O.k_mean_fixed_order(k, layout)
+    c = C.k_mean_fixed_order(k, layout)
+    assert a.dtype == dtype and a.shape == k.float().mean(dim=seq, keepdim=True).shape
+    assert torch.equal(a, c)
+    exact = k.double().mean(dim=seq, keepdim=True)
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    assert bool(((a.double() - exact).abs() <= ulp * exact.abs().clamp_min(2.0 ** -14)).all())
+    # constant rows: the mean is that constant exactly
+    kc = torch.full((1, 1, 256, 64), 1.25).to(dtype)
+    assert torch.equal(O.k_mean_fixed_order(kc), kc[:, :, :1])
+
+
+def test_config1_cpu_plumbing():
+    """B=1 H=2 N=256 D=64 fp16 HND, non-causal, smooth_k on: the whole path on CPU."""
+    g = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(1, 2, 256, 64, generator=g).to(torch.float16) for _ in range(3))
+    km = k.mean(dim=2, keepdim=True)
+    q8, qs, k8, ks = O.per_block_int8(q, k, km=km, sm_scale=1 / 8)
+    assert qs.shape == (1, 2, 2) and ks.shape == (1, 2, 4)
+    out, _ = O.attention_blockwise(q8, k8, v, qs, ks)
+    base = O.sdpa_cpu_baseline(q, k, v, output_dtype=torch.float16)
+    cos, rel, _ = O.accuracy_metrics(out, base)
+    assert cos >= 0.99 and rel <= 0.05  # the reference benchmark's own gate
