@@ -1,0 +1,4 @@
+"""``flag_attn.sage_attention`` namespace backed by ``flagattention_amd.sage_attention``."""
+from flagattention_amd.sage_attention import forward, k_mean, per_block_int8, sage_attention, sageattn
+
+__all__ = ["sage_attention", "forward", "per_block_int8", "k_mean", "sageattn"]

@@ -1,0 +1,449 @@
+// SageAttention forward for gfx950 (MI355X): INT8 Q.K^T on MFMA with int32 accumulation,
+// block-scale dequantization, fp32 online softmax (base 2), 16-bit P.V on MFMA.
+//
+// Replaces _attn_fwd / _attn_fwd_inner of FlagAttention
+// (src/flag_attn/sage_attention/attn_qk_int8_per_block.py:20-127).  Semantics kept: one q_scale
+// per 128 query rows and one k_scale per 64 keys (:42,115), scores = fp32(int32 dot) *
+// (q_scale * k_scale) (:44), masked / out-of-range scores get -1e6 added (:38,48,52), a 128x64
+// tile whose bool mask is False everywhere is skipped (:33-36), rows start at m = -inf, l = 1
+// (:110-111), lse = log2(l) + m (:126).
+//
+// Work decomposition (wave64, 32x32 MFMA tiles):
+//   workgroup = 4 waves = 128 query rows (one q_scale); wave w owns rows 32w .. 32w+31.
+//   Each KV step covers 64 keys (one k_scale).  The transposed products are computed,
+//       S^T[kv, q] = K . Q^T   (v_mfma_i32_32x32x32_i8,  A = K rows,   B = Q rows)
+//       O^T[d,  q] = V^T . P^T (v_mfma_f32_32x32x16_*,   A = V^T rows, B = P^T)
+//   so that every lane owns ONE query row (column q = lane % 32 of each accumulator tile): row
+//   max / row sum / alpha / q_scale are per-lane scalars, and the S^T accumulator registers are
+//   already laid out as the B operand of the P.V product (P never leaves registers).  The kv
+//   order inside an MFMA k-step is free as long as both operands agree; V^T is staged in LDS in
+//   exactly the order the S^T accumulator layout dictates (see v_chunk()).
+//   K tiles (int8 [64][D]) and V tiles (16-bit, transposed to [D][64]) are double buffered in LDS;
+//   global loads for step j+1 are issued before the math of step j.
+#include "common.h"
+
+namespace sage {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kThreads = 256;
+constexpr int BM = 128;  // query rows per workgroup (= Q quantization block)
+constexpr int BN = 64;   // keys per step (= K quantization block)
+constexpr float kMasked = -1.0e6f;
+
+enum { MODE_PLAIN = 0, MODE_CAUSAL = 1, MODE_MASK_BOOL = 2, MODE_MASK_F32 = 3 };
+
+struct AttnArgs {
+    const int8_t* q;
+    const int8_t* k;
+    const void* v;
+    void* out;
+    const float* q_scale;
+    const float* k_scale;
+    float* lse;
+    const void* mask;
+    int64_t qs_b, qs_h, qs_n;
+    int64_t ks_b, ks_h, ks_n;
+    int64_t vs_b, vs_h, vs_n;
+    int64_t os_b, os_h, os_n;
+    int64_t ms_b, ms_h, ms_m, ms_n;
+    int32_t Hq, Hkv, M, N, nq, nk, groups;
+    int32_t out_dt, causal;
+    int32_t total_wg;
+};
+
+template <typename VT> struct PV;
+template <> struct PV<__bf16> {
+    typedef bf16x8 vec;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct PV<_Float16> {
+    typedef f16x8 vec;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <int D>
+struct Tile {
+    static constexpr int KSTEPS = D / 32;           // int8 MFMA k-steps over head_dim
+    static constexpr int DTILES = D / 32;           // 32-row tiles of O^T
+    static constexpr int K_RS = D + 16;             // K tile row stride (bytes); +16 spreads rows over banks
+    static constexpr int K_BYTES = BN * K_RS;
+    static constexpr int V_RS = BN * 2;             // V^T row stride (bytes), XOR-swizzled 16-byte chunks
+    static constexpr int V_BYTES = D * V_RS;
+    static constexpr int STAGE = K_BYTES + V_BYTES;
+    static constexpr int K_CHUNKS_PER_ROW = D / 16;
+    static constexpr int K_LOADS = BN * K_CHUNKS_PER_ROW / kThreads;  // 16-byte loads per thread per K tile
+    static constexpr int V_ITEMS = (D / 8) * (BN / 4);                 // (8 channels x 4 keys) items per V tile
+};
+
+// XOR swizzle of the 16-byte chunk index inside a V^T row (row = channel d).
+__device__ __forceinline__ int v_swz(int d) { return (d ^ (d >> 3)) & 7; }
+
+// Chunk (16 bytes = 8 keys) and half-chunk (4 consecutive keys) that the run of keys
+// [4r, 4r+4) of a 64-key tile occupies in a V^T row.  The order is the one in which the S^T
+// accumulator hands P to the P.V MFMA: lane half h, k-step t' (16 keys each), slot c of 8 holds
+// key 16t' + 8(c/4) + 4h + c%4, i.e. run r = 4t' + 2(c/4) + h  ->  chunk 2t' + h, half c/4.
+__device__ __forceinline__ int v_chunk(int r) { return ((r >> 2) << 1) | (r & 1); }
+__device__ __forceinline__ int v_halfchunk(int r) { return (r >> 1) & 1; }
+
+__device__ __forceinline__ float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+__device__ __forceinline__ float xhalf_sum(float x) {
+    const float o = __shfl_xor(x, 32);
+    return (threadIdx.x & 32) ? (o + x) : (x + o);  // same operand order in both halves
+}
+
+template <int D, typename VT, int MODE>
+__global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) {
+    using T = Tile<D>;
+    using PVT = PV<VT>;
+    using vec16 = typename PVT::vec;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * T::STAGE];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+
+    // Workgroup -> (batch, head, q-block).  Consecutive workgroup ids land on different XCDs
+    // (8 of them, round robin); remap so that each XCD walks a contiguous range of logical ids and
+    // therefore keeps one head's K/V in its own L2 while it sweeps that head's q-blocks.
+    int wg = blockIdx.x;
+    {
+        const int per_xcd = a.total_wg >> 3;
+        if ((a.total_wg & 7) == 0) wg = (wg & 7) * per_xcd + (wg >> 3);
+    }
+    int iq = wg % a.nq;
+    if (MODE == MODE_CAUSAL) iq = a.nq - 1 - iq;  // longest rows first
+    const int h = (wg / a.nq) % a.Hq;
+    const int b = wg / (a.nq * a.Hq);
+    const int hk = h / a.groups;
+    const int m0 = iq * BM;
+    const int my_m = m0 + 32 * wave + l32;
+    const bool row_ok = my_m < a.M;
+
+    // ---- Q fragments (B operand of S^T = K.Q^T): lane (q = l32, half) holds channels
+    //      half*D/2 + 16t .. +15 for k-step t.  K fragments use the same channel order.
+    v4i qf[T::KSTEPS];
+    {
+        const int8_t* qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h + (int64_t)my_m * a.qs_n + half * (D / 2);
+#pragma unroll
+        for (int t = 0; t < T::KSTEPS; t++)
+            qf[t] = row_ok ? *reinterpret_cast<const v4i*>(qp + 16 * t) : v4i{0, 0, 0, 0};
+    }
+    const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + iq];
+    const float* ksp = a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk;
+
+    // ---- number of KV steps
+    int nsteps = a.nk;
+    if (MODE == MODE_CAUSAL || (MODE >= MODE_MASK_BOOL && a.causal)) {
+        // last visible column of the last valid row of this q-block
+        const int last_row = min(m0 + BM, a.M) - 1;
+        const int64_t hi = (int64_t)last_row + (a.N - a.M) + 1;  // exclusive
+        const int64_t hic = hi < (int64_t)a.N ? hi : (int64_t)a.N;
+        const int vis = hi <= 0 ? 0 : (int)((hic + BN - 1) / BN);
+        nsteps = min(nsteps, vis);
+    }
+
+    // ---- staging roles
+    const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
+    const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
+    int k_row[T::K_LOADS], k_lds[T::K_LOADS], k_goff[T::K_LOADS];
+#pragma unroll
+    for (int j = 0; j < T::K_LOADS; j++) {
+        const int id = tid + kThreads * j;
+        k_row[j] = id / T::K_CHUNKS_PER_ROW;
+        const int c = id % T::K_CHUNKS_PER_ROW;
+        k_lds[j] = k_row[j] * T::K_RS + 16 * c;
+        k_goff[j] = 16 * c;
+    }
+    const bool v_worker = tid < T::V_ITEMS;
+    const int v_dg = tid % (D / 8);  // group of 8 channels
+    const int v_r = tid / (D / 8);   // run of 4 keys
+    int v_lds[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const int d = 8 * v_dg + e;
+        v_lds[e] = T::K_BYTES + d * T::V_RS + ((v_chunk(v_r) ^ v_swz(d)) * 16) + v_halfchunk(v_r) * 8;
+    }
+
+    v4i kreg[T::K_LOADS];
+    uint4 vreg[4];
+    auto load_tile = [&](int step) {
+        const int n0 = step * BN;
+#pragma unroll
+        for (int j = 0; j < T::K_LOADS; j++) {
+            const int n = n0 + k_row[j];
+            kreg[j] = (n < a.N) ? *reinterpret_cast<const v4i*>(kg + (int64_t)n * a.ks_n + k_goff[j]) : v4i{0, 0, 0, 0};
+        }
+        if (v_worker) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int n = n0 + 4 * v_r + i;
+                vreg[i] = (n < a.N) ? *reinterpret_cast<const uint4*>(vg + (int64_t)n * a.vs_n + 8 * v_dg)
+                                    : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+        unsigned char* base = smem + buf * T::STAGE;
+#pragma unroll
+        for (int j = 0; j < T::K_LOADS; j++) *reinterpret_cast<v4i*>(base + k_lds[j]) = kreg[j];
+        if (v_worker) {
+            const uint32_t r0[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
+            const uint32_t r1[4] = {vreg[1].x, vreg[1].y, vreg[1].z, vreg[1].w};
+            const uint32_t r2[4] = {vreg[2].x, vreg[2].y, vreg[2].z, vreg[2].w};
+            const uint32_t r3[4] = {vreg[3].x, vreg[3].y, vreg[3].z, vreg[3].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                // channel 2i (low halves) and 2i+1 (high halves) of four consecutive keys
+                uint2 lo, hi;
+                lo.x = __builtin_amdgcn_perm(r1[i], r0[i], 0x05040100u);
+                lo.y = __builtin_amdgcn_perm(r3[i], r2[i], 0x05040100u);
+                hi.x = __builtin_amdgcn_perm(r1[i], r0[i], 0x07060302u);
+                hi.y = __builtin_amdgcn_perm(r3[i], r2[i], 0x07060302u);
+                *reinterpret_cast<uint2*>(base + v_lds[2 * i]) = lo;
+                *reinterpret_cast<uint2*>(base + v_lds[2 * i + 1]) = hi;
+            }
+        }
+    };
+
+    // ---- per-lane LDS read offsets
+    const int kf_off = l32 * T::K_RS + 16 * half * (D / 32);
+    int vf_off[4];
+    {
+        const int x0 = (half ^ v_swz(l32)) & 7;
+#pragma unroll
+        for (int i = 0; i < 4; i++) vf_off[i] = T::K_BYTES + l32 * T::V_RS + (((2 * i) ^ x0) * 16);
+    }
+
+    // ---- running state: this lane's query row
+    float m_i = -INFINITY;
+    float l_i = half ? 0.0f : 1.0f;  // the two halves of a row sum to the reference's l = 1
+    v16f o[T::DTILES];
+#pragma unroll
+    for (int dt = 0; dt < T::DTILES; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+
+    if (nsteps > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int step = 0; step < nsteps; step++) {
+        const int buf = step & 1;
+        const bool more = step + 1 < nsteps;
+        if (more) load_tile(step + 1);
+        const unsigned char* base = smem + buf * T::STAGE;
+        const int n0 = step * BN;
+
+        // generic masks: fetch this lane's 32 mask entries, decide the tile skip (bool only)
+        float madd[2][16];
+        bool skip = false;
+        if (MODE >= MODE_MASK_BOOL) {
+            const int64_t mrow = (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)my_m * a.ms_m;
+            int any = 0;
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
+                    const bool inb = row_ok && n < a.N;
+                    bool keep = inb;
+                    if (a.causal) keep = keep && (n <= my_m + (a.N - a.M));
+                    if (MODE == MODE_MASK_BOOL) {
+                        if (keep) keep = static_cast<const uint8_t*>(a.mask)[mrow + (int64_t)n * a.ms_n] != 0;
+                        madd[kt][i] = keep ? 0.0f : kMasked;
+                        any |= keep;
+                    } else {
+                        float add = inb ? static_cast<const float*>(a.mask)[mrow + (int64_t)n * a.ms_n] : kMasked;
+                        if (a.causal && inb && !keep) add += kMasked;
+                        madd[kt][i] = add;
+                        any |= keep;
+                    }
+                }
+            if (MODE == MODE_MASK_BOOL || a.causal) skip = !__syncthreads_or(any);
+        }
+
+        if (!skip) {
+            // ---- S^T = K . Q^T
+            v16i sacc[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) sacc[kt][i] = 0;
+#pragma unroll
+                for (int t = 0; t < T::KSTEPS; t++) {
+                    const v4i kf = *reinterpret_cast<const v4i*>(base + kf_off + 32 * kt * T::K_RS + 16 * t);
+                    sacc[kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[t], sacc[kt], 0, 0, 0);
+                }
+            }
+
+            // ---- online softmax (base 2), one row per lane
+            const float sc = qs * ksp[step];
+            float s[2][16];
+            float rmax = -INFINITY;
+            bool plain = (MODE == MODE_PLAIN) && (n0 + BN <= a.N);
+            if (MODE == MODE_CAUSAL) plain = (n0 + BN <= a.N) && (n0 + BN - 1 <= m0 + 32 * wave + (a.N - a.M));
+            if (plain) {
+                // no element needs masking: fold the dequantization into the exponent's fma
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        s[kt][i] = (float)sacc[kt][i];
+                        rmax = fmaxf(rmax, s[kt][i]);
+                    }
+                rmax = xhalf_max(rmax) * sc;
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        float x = (float)sacc[kt][i] * sc;
+                        if (MODE >= MODE_MASK_BOOL) {
+                            x += madd[kt][i];
+                        } else {
+                            const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
+                            bool keep = n < a.N;
+                            if (MODE == MODE_CAUSAL) keep = keep && (n <= my_m + (a.N - a.M));
+                            x += keep ? 0.0f : kMasked;
+                        }
+                        s[kt][i] = x;
+                        rmax = fmaxf(rmax, x);
+                    }
+                rmax = xhalf_max(rmax);
+            }
+            const float m_new = fmaxf(m_i, rmax);
+            const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+            float lsum = 0.0f;
+            if (plain) {
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        s[kt][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], sc, -m_new));
+                        lsum += s[kt][i];
+                    }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        s[kt][i] = __builtin_amdgcn_exp2f(s[kt][i] - m_new);
+                        lsum += s[kt][i];
+                    }
+            }
+            l_i = l_i * alpha + lsum;
+            m_i = m_new;
+#pragma unroll
+            for (int dt = 0; dt < T::DTILES; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+
+            // ---- P^T as the B operand: k-step t' of 16 keys takes S^T registers 8(t'&1) .. +7 of tile t'>>1
+            vec16 pf[4];
+#pragma unroll
+            for (int tp = 0; tp < 4; tp++)
+#pragma unroll
+                for (int c = 0; c < 8; c++) pf[tp][c] = (VT)s[tp >> 1][8 * (tp & 1) + c];
+
+            // ---- O^T += V^T . P^T
+#pragma unroll
+            for (int dt = 0; dt < T::DTILES; dt++)
+#pragma unroll
+                for (int tp = 0; tp < 4; tp++) {
+                    const vec16 vf = *reinterpret_cast<const vec16*>(base + vf_off[tp ^ (2 * (dt & 1))] + dt * 32 * T::V_RS);
+                    o[dt] = PVT::mfma(vf, pf[tp], o[dt]);
+                }
+        }
+
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: O = O^T / l, lse = log2(l) + m
+    const float l_tot = xhalf_sum(l_i);
+    const float inv = 1.0f / l_tot;
+    if (row_ok) {
+        const int64_t obase = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)my_m * a.os_n;
+#pragma unroll
+        for (int dt = 0; dt < T::DTILES; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = 32 * dt + 8 * g + 4 * half;
+                float r[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] = o[dt][4 * g + i] * inv;
+                if (a.out_dt == SAGE_BF16) {
+                    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+                    b4 w = {(__bf16)r[0], (__bf16)r[1], (__bf16)r[2], (__bf16)r[3]};
+                    *reinterpret_cast<b4*>(static_cast<__bf16*>(a.out) + obase + d) = w;
+                } else if (a.out_dt == SAGE_F16) {
+                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                    h4 w = {(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
+                    *reinterpret_cast<h4*>(static_cast<_Float16*>(a.out) + obase + d) = w;
+                } else {
+                    *reinterpret_cast<v4f*>(static_cast<float*>(a.out) + obase + d) = v4f{r[0], r[1], r[2], r[3]};
+                }
+            }
+        if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
+    }
+}
+
+template <int D, typename VT>
+int launch_mode(const AttnArgs& a, int mode, hipStream_t stream) {
+    dim3 grid((unsigned)a.total_wg), block(kThreads);
+    switch (mode) {
+        case MODE_PLAIN: hipLaunchKernelGGL((sage_attn_fwd_kernel<D, VT, MODE_PLAIN>), grid, block, 0, stream, a); break;
+        case MODE_CAUSAL: hipLaunchKernelGGL((sage_attn_fwd_kernel<D, VT, MODE_CAUSAL>), grid, block, 0, stream, a); break;
+        case MODE_MASK_BOOL: hipLaunchKernelGGL((sage_attn_fwd_kernel<D, VT, MODE_MASK_BOOL>), grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((sage_attn_fwd_kernel<D, VT, MODE_MASK_F32>), grid, block, 0, stream, a); break;
+    }
+    return check_launch("sage_attn_fwd_kernel");
+}
+
+}  // namespace
+
+int launch_attn(const sage_attn_params& p, hipStream_t stream) {
+    AttnArgs a{};
+    a.q = (const int8_t*)p.q.ptr; a.k = (const int8_t*)p.k.ptr; a.v = p.v.ptr; a.out = p.out.ptr;
+    a.q_scale = p.q_scale; a.k_scale = p.k_scale; a.lse = p.lse; a.mask = p.mask;
+    a.qs_b = p.q.stride_b; a.qs_h = p.q.stride_h; a.qs_n = p.q.stride_n;
+    a.ks_b = p.k.stride_b; a.ks_h = p.k.stride_h; a.ks_n = p.k.stride_n;
+    a.vs_b = p.v.stride_b; a.vs_h = p.v.stride_h; a.vs_n = p.v.stride_n;
+    a.os_b = p.out.stride_b; a.os_h = p.out.stride_h; a.os_n = p.out.stride_n;
+    a.ms_b = p.mask_stride_b; a.ms_h = p.mask_stride_h; a.ms_m = p.mask_stride_m; a.ms_n = p.mask_stride_n;
+    a.Hq = (int)p.heads_q; a.Hkv = (int)p.heads_kv; a.M = (int)p.qo_len; a.N = (int)p.kv_len;
+    a.nq = (int)((p.qo_len + BM - 1) / BM); a.nk = (int)((p.kv_len + BN - 1) / BN);
+    a.groups = (int)(p.heads_q / p.heads_kv);
+    a.out_dt = p.out_dtype; a.causal = p.causal ? 1 : 0;
+    const int64_t total = p.batch * p.heads_q * a.nq;
+    if (total > 0x7fffffffLL || p.qo_len > 0x7fffffffLL - BM || p.kv_len > 0x7fffffffLL - BN)
+        return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: problem too large for 32-bit tile indices");
+    a.total_wg = (int)total;
+    int mode = MODE_PLAIN;
+    if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
+    else if (p.mask_kind == SAGE_MASK_F32) mode = MODE_MASK_F32;
+    else if (p.causal) mode = MODE_CAUSAL;
+    if (p.head_dim == 128) {
+        return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)
+                                      : launch_mode<128, _Float16>(a, mode, stream);
+    }
+    return p.v_dtype == SAGE_BF16 ? launch_mode<64, __bf16>(a, mode, stream)
+                                  : launch_mode<64, _Float16>(a, mode, stream);
+}
+
+}  // namespace sage

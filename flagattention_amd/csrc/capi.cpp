@@ -1,0 +1,96 @@
+// extern "C" surface of libsage_attention_hip.so: argument validation and dispatch only.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+namespace sage {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static bool float_dtype_ok(int dt) { return dt == SAGE_F16 || dt == SAGE_BF16 || dt == SAGE_F32; }
+
+}  // namespace sage
+
+using namespace sage;
+
+extern "C" const char* sage_hip_last_error(void) { return g_err; }
+extern "C" int sage_hip_abi_version(void) { return SAGE_HIP_ABI_VERSION; }
+
+extern "C" int sage_per_block_int8(const sage_quant_params* p, void* stream) {
+    if (!p) return fail(SAGE_E_INVALID, "sage_per_block_int8: null params");
+    if (p->batch < 0 || p->heads_q < 0 || p->heads_kv < 0 || p->qo_len < 0 || p->kv_len < 0)
+        return fail(SAGE_E_INVALID, "sage_per_block_int8: negative size");
+    if (p->head_dim <= 0 || p->head_dim % 8 != 0)
+        return fail(SAGE_E_UNSUPPORTED, "sage_per_block_int8: head_dim %lld must be a positive multiple of 8",
+                    (long long)p->head_dim);
+    if (!float_dtype_ok(p->in_dtype)) return fail(SAGE_E_INVALID, "sage_per_block_int8: bad in_dtype %d", p->in_dtype);
+    if (p->q.ptr && (p->blkq <= 0 || (int64_t)p->blkq * p->head_dim > 32768))
+        return fail(SAGE_E_UNSUPPORTED, "sage_per_block_int8: BLKQ*head_dim = %lld exceeds 32768",
+                    (long long)p->blkq * p->head_dim);
+    if (p->k.ptr && (p->blkk <= 0 || (int64_t)p->blkk * p->head_dim > 32768))
+        return fail(SAGE_E_UNSUPPORTED, "sage_per_block_int8: BLKK*head_dim = %lld exceeds 32768",
+                    (long long)p->blkk * p->head_dim);
+    if (p->q.ptr && (!p->q_int8.ptr || !p->q_scale)) return fail(SAGE_E_INVALID, "sage_per_block_int8: null Q output");
+    if (p->k.ptr && (!p->k_int8.ptr || !p->k_scale)) return fail(SAGE_E_INVALID, "sage_per_block_int8: null K output");
+    if (p->km.ptr) {
+        if (!float_dtype_ok(p->km_dtype) || !float_dtype_ok(p->diff_dtype))
+            return fail(SAGE_E_INVALID, "sage_per_block_int8: bad km_dtype/diff_dtype");
+        if (p->in_dtype == SAGE_F32 && p->diff_dtype != SAGE_F32)
+            return fail(SAGE_E_INVALID, "sage_per_block_int8: fp32 K needs diff_dtype fp32");
+    }
+    return launch_quant(*p, (hipStream_t)stream);
+}
+
+extern "C" int64_t sage_k_mean_workspace_bytes(int64_t batch, int64_t heads_kv, int64_t kv_len, int64_t head_dim) {
+    int64_t nchunk = (kv_len + 63) / 64;
+    return batch * heads_kv * nchunk * head_dim * (int64_t)sizeof(float);
+}
+
+extern "C" int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out_dtype, int64_t batch,
+                           int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* workspace, void* stream) {
+    if (!k || !k->ptr || !km_out || !workspace) return fail(SAGE_E_INVALID, "sage_k_mean: null pointer");
+    if (!float_dtype_ok(k_dtype) || !float_dtype_ok(out_dtype)) return fail(SAGE_E_INVALID, "sage_k_mean: bad dtype");
+    if (batch <= 0 || heads_kv <= 0 || kv_len <= 0 || head_dim <= 0)
+        return fail(SAGE_E_INVALID, "sage_k_mean: sizes must be positive");
+    return launch_kmean(*k, k_dtype, km_out, out_dtype, batch, heads_kv, kv_len, head_dim, workspace,
+                        (hipStream_t)stream);
+}
+
+extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
+    if (!p) return fail(SAGE_E_INVALID, "sage_attn_fwd: null params");
+    if (!p->q.ptr || !p->k.ptr || !p->v.ptr || !p->out.ptr || !p->q_scale || !p->k_scale)
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: null tensor pointer");
+    if (p->head_dim != 64 && p->head_dim != 128)
+        return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: head_dim %lld not supported (64 or 128)",
+                    (long long)p->head_dim);
+    if (p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->qo_len <= 0 || p->kv_len <= 0)
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: sizes must be positive");
+    if (p->heads_q % p->heads_kv != 0)
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: heads_q %lld is not a multiple of heads_kv %lld",
+                    (long long)p->heads_q, (long long)p->heads_kv);
+    if (p->v_dtype != SAGE_F16 && p->v_dtype != SAGE_BF16)
+        return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: V must be fp16 or bf16");
+    if (!float_dtype_ok(p->out_dtype)) return fail(SAGE_E_INVALID, "sage_attn_fwd: bad out_dtype %d", p->out_dtype);
+    if (p->mask_kind != SAGE_MASK_NONE && p->mask_kind != SAGE_MASK_BOOL && p->mask_kind != SAGE_MASK_F32)
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: bad mask_kind %d", p->mask_kind);
+    if (p->mask_kind != SAGE_MASK_NONE && !p->mask) return fail(SAGE_E_INVALID, "sage_attn_fwd: null mask");
+    // 16-byte vector loads: row starts of Q/K (int8) and V (16-bit) must be 16-byte aligned
+    auto misaligned = [](const sage_tensor& t, int esz) {
+        return ((uintptr_t)t.ptr % 16) != 0 || (t.stride_b * esz) % 16 != 0 || (t.stride_h * esz) % 16 != 0 ||
+               (t.stride_n * esz) % 16 != 0;
+    };
+    if (misaligned(p->q, 1) || misaligned(p->k, 1) || misaligned(p->v, 2))
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: q/k/v rows must be 16-byte aligned");
+    if (misaligned(p->out, dtype_bytes(p->out_dtype)))
+        return fail(SAGE_E_INVALID, "sage_attn_fwd: out rows must be 16-byte aligned");
+    return launch_attn(*p, (hipStream_t)stream);
+}

@@ -1,0 +1,27 @@
+// Shared host-side helpers of libsage_attention_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/sage_attention_hip.h"
+
+namespace sage {
+
+// Records a printf-style message for sage_hip_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+inline int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SAGE_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return SAGE_OK;
+}
+
+inline int dtype_bytes(int dt) { return dt == SAGE_F32 ? 4 : 2; }
+
+// Launchers implemented in the .hip files.
+int launch_quant(const sage_quant_params& p, hipStream_t stream);
+int launch_kmean(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype, int64_t B, int64_t H, int64_t N,
+                 int64_t D, void* workspace, hipStream_t stream);
+int launch_attn(const sage_attn_params& p, hipStream_t stream);
+
+}  // namespace sage

@@ -1,0 +1,332 @@
+// Per-block INT8 quantization of Q and K (with the `k - km` smoothing fused in) and the
+// fixed-order K mean, for gfx950.
+//
+// Arithmetic follows quant_per_block_int8_kernel (FlagAttention
+// src/flag_attn/sage_attention/quant_per_block.py:38-46) operation by operation in IEEE fp32:
+//   x = fp32(in) [* sm_scale];  scale = max|x| / 127;  y = x / scale;  y += (y >= 0 ? .5 : -.5);
+//   q = (int8) truncate(y)
+// and `k - km` (:53-54) is one fp32 subtraction rounded once to the promoted dtype.
+//
+// HBM-bound: one workgroup per [BLK, D] block reads the block once (16-byte loads, coalesced
+// along head_dim), keeps it in registers as fp32, reduces max|x| with wave shuffles plus one LDS
+// step, and writes 8-byte int8 groups.  Algorithmic traffic: in_bytes + 1 byte per element.
+#include "common.h"
+
+namespace sage {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct QuantArgs {
+    const void* x;
+    const void* km;
+    int8_t* out;
+    float* scale;
+    int64_t xs_b, xs_h, xs_n;
+    int64_t ks_b, ks_h, ks_n;
+    int64_t os_b, os_h, os_n;
+    int32_t H, L, D8, d8_shift, blk, nblk;
+    int32_t km_dt, diff_dt;
+    int32_t apply_mul;
+    float mul;
+};
+
+__device__ __forceinline__ void unpack8(const uint4& r, int dt, float (&v)[8]) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+    if (dt == SAGE_BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+            v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xffffu));
+            v[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+        }
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t elem_off, float (&v)[8]) {
+    if constexpr (DT == SAGE_F32) {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(base) + elem_off);
+        float4 a = p[0], b = p[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        uint4 r = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + elem_off);
+        unpack8(r, DT, v);
+    }
+}
+
+__device__ __forceinline__ void load8_rt(const void* base, int dt, int64_t elem_off, float (&v)[8]) {
+    if (dt == SAGE_F32) load8<SAGE_F32>(base, elem_off, v);
+    else if (dt == SAGE_BF16) load8<SAGE_BF16>(base, elem_off, v);
+    else load8<SAGE_F16>(base, elem_off, v);
+}
+
+__device__ __forceinline__ float round_to(float x, int dt) {
+    if (dt == SAGE_BF16) return (float)(__bf16)x;
+    if (dt == SAGE_F16) return (float)(_Float16)x;
+    return x;
+}
+
+// One workgroup = one quantization block of `blk` rows; UNITS 8-element groups per thread.
+template <int DT, int UNITS>
+__global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArgs a) {
+    const int tid = threadIdx.x;
+    const int bid = blockIdx.x;
+    const int ib = bid % a.nblk;
+    const int h = (bid / a.nblk) % a.H;
+    const int b = bid / (a.nblk * a.H);
+    const int total_units = a.blk * a.D8;
+
+    const int64_t x_base = (int64_t)b * a.xs_b + (int64_t)h * a.xs_h;
+    const int64_t o_base = (int64_t)b * a.os_b + (int64_t)h * a.os_h;
+    const int64_t k_base = (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
+
+    float v[UNITS][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < UNITS; j++) {
+        const int u = tid + kThreads * j;
+        int row, c8;
+        if (a.d8_shift >= 0) {
+            row = u >> a.d8_shift;
+            c8 = u & (a.D8 - 1);
+        } else {
+            row = u / a.D8;
+            c8 = u - row * a.D8;
+        }
+        const int n = ib * a.blk + row;
+        const bool live = (u < total_units) && (n < a.L);
+        if (live) {
+            load8<DT>(a.x, x_base + (int64_t)n * a.xs_n + c8 * 8, v[j]);
+            if (a.km) {
+                float m[8];
+                load8_rt(a.km, a.km_dt, k_base + (int64_t)n * a.ks_n + c8 * 8, m);
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[j][e] = round_to(v[j][e] - m[e], a.diff_dt);
+            }
+            if (a.apply_mul) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[j][e] = v[j][e] * a.mul;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[j][e] = 0.0f;  // rows past L are masked loads: zeros
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[j][e]));
+    }
+
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    __shared__ float wave_max[kThreads / 64];
+    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+
+    const float scale = amax / 127.0f;
+    if (tid == 0) a.scale[((int64_t)b * a.H + h) * a.nblk + ib] = scale;
+    const bool zero_block = !(scale > 0.0f);  // 0/0 -> NaN in the reference; its int8 conversion yields 0
+
+#pragma unroll
+    for (int j = 0; j < UNITS; j++) {
+        const int u = tid + kThreads * j;
+        int row, c8;
+        if (a.d8_shift >= 0) {
+            row = u >> a.d8_shift;
+            c8 = u & (a.D8 - 1);
+        } else {
+            row = u / a.D8;
+            c8 = u - row * a.D8;
+        }
+        const int n = ib * a.blk + row;
+        if ((u < total_units) && (n < a.L)) {
+            uint32_t packed[2] = {0u, 0u};
+            if (!zero_block) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    float y = v[j][e] / scale;  // IEEE fp32 divide (hipcc default is correctly rounded)
+                    y = y + (y >= 0.0f ? 0.5f : -0.5f);
+                    const int q = (int)y;  // truncation toward zero; |y| <= 127.5
+                    packed[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
+                }
+            }
+            *reinterpret_cast<uint2*>(a.out + o_base + (int64_t)n * a.os_n + c8 * 8) = make_uint2(packed[0], packed[1]);
+        }
+    }
+}
+
+template <int DT>
+int launch_one(const QuantArgs& a, int64_t nblocks, hipStream_t stream) {
+    const int total_units = a.blk * a.D8;
+    const int units = (total_units + kThreads - 1) / kThreads;
+    dim3 grid((unsigned)nblocks), block(kThreads);
+    if (units <= 1) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1>), grid, block, 0, stream, a);
+    else if (units <= 2) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 2>), grid, block, 0, stream, a);
+    else if (units <= 4) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 4>), grid, block, 0, stream, a);
+    else if (units <= 8) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 8>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 16>), grid, block, 0, stream, a);
+    return check_launch("quant_per_block_int8_kernel");
+}
+
+int launch_tensor(const QuantArgs& a, int in_dtype, int64_t nblocks, hipStream_t stream) {
+    if (nblocks <= 0) return SAGE_OK;
+    if (nblocks > 0x7fffffffLL) return fail(SAGE_E_UNSUPPORTED, "sage_per_block_int8: too many blocks");
+    switch (in_dtype) {
+        case SAGE_F16: return launch_one<SAGE_F16>(a, nblocks, stream);
+        case SAGE_BF16: return launch_one<SAGE_BF16>(a, nblocks, stream);
+        default: return launch_one<SAGE_F32>(a, nblocks, stream);
+    }
+}
+
+bool aligned_to(int align, const void* p, int esz, int64_t s0, int64_t s1, int64_t s2) {
+    return ((uintptr_t)p % align) == 0 && (s0 * esz) % align == 0 && (s1 * esz) % align == 0 &&
+           (s2 * esz) % align == 0;
+}
+bool aligned16(const void* p, int esz, int64_t s0, int64_t s1, int64_t s2) {
+    return aligned_to(16, p, esz, s0, s1, s2);
+}
+
+// ---------------------------------------------------------------------------------------------
+// K mean, fixed order.  Stage 1: one thread per (chunk of 64 rows, 8 channels) adds the rows in
+// order.  Stage 2: one thread per channel adds the chunk partials in order, divides, rounds.
+// ---------------------------------------------------------------------------------------------
+struct KMeanArgs {
+    const void* k;
+    float* part;  // [B*H, nchunk, D]
+    void* out;    // [B*H, D]
+    int64_t s_b, s_h, s_n;
+    int32_t H, N, D, D8, nchunk, out_dt;
+    int64_t total_items;  // B*H*nchunk*D8
+};
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void k_mean_partial_kernel(KMeanArgs a) {
+    const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (item >= a.total_items) return;
+    const int c8 = (int)(item % a.D8);
+    const int64_t t = item / a.D8;
+    const int chunk = (int)(t % a.nchunk);
+    const int64_t bh = t / a.nchunk;
+    const int h = (int)(bh % a.H);
+    const int64_t b = bh / a.H;
+    const int64_t base = b * a.s_b + (int64_t)h * a.s_h + c8 * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int n0 = chunk * 64;
+    const int rows = min(64, a.N - n0);
+    int r = 0;
+    for (; r + 8 <= rows; r += 8) {
+        float v[8][8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) load8<DT>(a.k, base + (int64_t)(n0 + r + i) * a.s_n, v[i]);
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] = acc[e] + v[i][e];
+    }
+    for (; r < rows; r++) {
+        float v[8];
+        load8<DT>(a.k, base + (int64_t)(n0 + r) * a.s_n, v);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = acc[e] + v[e];
+    }
+    float4* dst = reinterpret_cast<float4*>(a.part + (bh * a.nchunk + chunk) * a.D + c8 * 8);
+    dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
+
+__global__ __launch_bounds__(kThreads) void k_mean_final_kernel(KMeanArgs a, int64_t channels) {
+    const int64_t ch = (int64_t)blockIdx.x * kThreads + threadIdx.x;  // (b*H + h) * D + d
+    if (ch >= channels) return;
+    const int64_t bh = ch / a.D;
+    const int d = (int)(ch % a.D);
+    const float* p = a.part + bh * a.nchunk * a.D + d;
+    float tot = 0.0f;
+    for (int c = 0; c < a.nchunk; c++) tot = tot + p[(int64_t)c * a.D];
+    const float mean = tot / (float)a.N;
+    if (a.out_dt == SAGE_F32) static_cast<float*>(a.out)[ch] = mean;
+    else if (a.out_dt == SAGE_BF16) static_cast<__bf16*>(a.out)[ch] = (__bf16)mean;
+    else static_cast<_Float16*>(a.out)[ch] = (_Float16)mean;
+}
+
+}  // namespace
+
+int launch_quant(const sage_quant_params& p, hipStream_t stream) {
+    const int esz = dtype_bytes(p.in_dtype);
+    const int64_t D = p.head_dim;
+    int shift = -1;
+    const int D8 = (int)(D / 8);
+    if ((D8 & (D8 - 1)) == 0) {
+        shift = 0;
+        while ((1 << shift) < D8) shift++;
+    }
+    if (p.q.ptr && p.qo_len > 0) {
+        if (!aligned16(p.q.ptr, esz, p.q.stride_b, p.q.stride_h, p.q.stride_n) ||
+            !aligned_to(8, p.q_int8.ptr, 1, p.q_int8.stride_b, p.q_int8.stride_h, p.q_int8.stride_n))
+            return fail(SAGE_E_INVALID, "sage_per_block_int8: q rows must be 16-byte aligned (8-byte for int8 output)");
+        QuantArgs a{};
+        a.x = p.q.ptr; a.km = nullptr; a.out = (int8_t*)p.q_int8.ptr; a.scale = p.q_scale;
+        a.xs_b = p.q.stride_b; a.xs_h = p.q.stride_h; a.xs_n = p.q.stride_n;
+        a.os_b = p.q_int8.stride_b; a.os_h = p.q_int8.stride_h; a.os_n = p.q_int8.stride_n;
+        a.H = (int)p.heads_q; a.L = (int)p.qo_len; a.D8 = D8; a.d8_shift = shift; a.blk = p.blkq;
+        a.nblk = (int)((p.qo_len + p.blkq - 1) / p.blkq);
+        a.apply_mul = (p.q_mul != 1.0f); a.mul = p.q_mul;
+        int rc = launch_tensor(a, p.in_dtype, p.batch * p.heads_q * a.nblk, stream);
+        if (rc) return rc;
+    }
+    if (p.k.ptr && p.kv_len > 0) {
+        if (!aligned16(p.k.ptr, esz, p.k.stride_b, p.k.stride_h, p.k.stride_n) ||
+            !aligned_to(8, p.k_int8.ptr, 1, p.k_int8.stride_b, p.k_int8.stride_h, p.k_int8.stride_n))
+            return fail(SAGE_E_INVALID, "sage_per_block_int8: k rows must be 16-byte aligned (8-byte for int8 output)");
+        QuantArgs a{};
+        a.x = p.k.ptr; a.out = (int8_t*)p.k_int8.ptr; a.scale = p.k_scale;
+        a.xs_b = p.k.stride_b; a.xs_h = p.k.stride_h; a.xs_n = p.k.stride_n;
+        a.os_b = p.k_int8.stride_b; a.os_h = p.k_int8.stride_h; a.os_n = p.k_int8.stride_n;
+        if (p.km.ptr) {
+            if (!aligned16(p.km.ptr, dtype_bytes(p.km_dtype), p.km.stride_b, p.km.stride_h, p.km.stride_n))
+                return fail(SAGE_E_INVALID, "sage_per_block_int8: km rows must be 16-byte aligned");
+            a.km = p.km.ptr; a.ks_b = p.km.stride_b; a.ks_h = p.km.stride_h; a.ks_n = p.km.stride_n;
+            a.km_dt = p.km_dtype; a.diff_dt = p.diff_dtype;
+        }
+        a.H = (int)p.heads_kv; a.L = (int)p.kv_len; a.D8 = D8; a.d8_shift = shift; a.blk = p.blkk;
+        a.nblk = (int)((p.kv_len + p.blkk - 1) / p.blkk);
+        a.apply_mul = 0; a.mul = 1.0f;
+        int rc = launch_tensor(a, p.in_dtype, p.batch * p.heads_kv * a.nblk, stream);
+        if (rc) return rc;
+    }
+    return SAGE_OK;
+}
+
+int launch_kmean(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype, int64_t B, int64_t H, int64_t N,
+                 int64_t D, void* workspace, hipStream_t stream) {
+    if (D % 8 != 0) return fail(SAGE_E_UNSUPPORTED, "sage_k_mean: head_dim must be a multiple of 8");
+    if (!aligned16(k.ptr, dtype_bytes(k_dtype), k.stride_b, k.stride_h, k.stride_n) || ((uintptr_t)workspace % 16))
+        return fail(SAGE_E_INVALID, "sage_k_mean: k rows and workspace must be 16-byte aligned");
+    KMeanArgs a{};
+    a.k = k.ptr; a.part = (float*)workspace; a.out = km_out;
+    a.s_b = k.stride_b; a.s_h = k.stride_h; a.s_n = k.stride_n;
+    a.H = (int)H; a.N = (int)N; a.D = (int)D; a.D8 = (int)(D / 8); a.nchunk = (int)((N + 63) / 64);
+    a.out_dt = out_dtype;
+    a.total_items = B * H * a.nchunk * a.D8;
+    const int64_t g1 = (a.total_items + kThreads - 1) / kThreads;
+    const int64_t channels = B * H * D;
+    const int64_t g2 = (channels + kThreads - 1) / kThreads;
+    if (g1 > 0x7fffffffLL) return fail(SAGE_E_UNSUPPORTED, "sage_k_mean: too many chunks");
+    dim3 block(kThreads);
+    switch (k_dtype) {
+        case SAGE_F16: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_F16>, dim3((unsigned)g1), block, 0, stream, a); break;
+        case SAGE_BF16: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_BF16>, dim3((unsigned)g1), block, 0, stream, a); break;
+        default: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_F32>, dim3((unsigned)g1), block, 0, stream, a); break;
+    }
+    int rc = check_launch("k_mean_partial_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)g2), block, 0, stream, a, channels);
+    return check_launch("k_mean_final_kernel");
+}
+
+}  // namespace sage

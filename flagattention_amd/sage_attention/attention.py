@@ -1,0 +1,114 @@
+"""``forward`` / ``sage_attention``: INT8-QK flash attention forward on MI355X.
+
+Host side of FlagAttention's src/flag_attn/sage_attention/attn_qk_int8_per_block.py:129-191 with
+the same positional signature, defaults, return convention and errors.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .. import _lib
+from ._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, tensor_desc
+
+BLOCK_M = 128  # attn_qk_int8_per_block.py:131
+BLOCK_N = 64  # attn_qk_int8_per_block.py:132
+
+
+def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
+            output_dtype=torch.float16, return_lse=False, maxnreg=None, *, causal=False):
+    """``(o, lse)`` like the reference: ``o`` has ``q``'s shape and ``output_dtype``; ``lse`` is the
+    base-2 log-sum-exp ``[B, Hq, M]`` fp32 when ``return_lse`` else an empty fp32 CPU tensor.
+
+    ``q`` / ``k`` are the int8 tensors and ``q_scale`` / ``k_scale`` the fp32 block scales that
+    ``per_block_int8`` (BLKQ=128, BLKK=64) returns; ``v`` is fp16 or bf16.  ``attn_mask`` is a
+    bool (True = keep) or additive mask broadcastable to ``[B, Hq, M, N]``.  ``maxnreg`` is a
+    register cap for the reference's Triton launch: validated, otherwise ignored.
+    ``causal=True`` (keyword only, not in the reference) applies the bottom-right aligned causal
+    mask ``n <= m + (N - M)`` with whole-tile skipping.
+    """
+    if tensor_layout not in ("HND", "NHD"):
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    if maxnreg is not None and maxnreg <= 0:
+        raise ValueError("maxnreg must be positive")
+    hnd = tensor_layout == "HND"
+    for name, t in (("q", q), ("k", k), ("v", v), ("q_scale", q_scale), ("k_scale", k_scale)):
+        require_gpu(t, name)
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k and v must be 4-D")
+    if q.dtype != torch.int8 or k.dtype != torch.int8:
+        raise TypeError(f"q and k must be int8 (per_block_int8 outputs), got {q.dtype} and {k.dtype}")
+    if v.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"v must be float16 or bfloat16, got {v.dtype}")
+    if output_dtype not in DTYPE_CODE:
+        raise TypeError(f"output_dtype {output_dtype} not supported (float16, bfloat16, float32)")
+    if hnd:
+        b, h_qo, qo_len, head_dim = q.shape
+        _, h_kv, kv_len, _ = k.shape
+    else:
+        b, qo_len, h_qo, head_dim = q.shape
+        _, kv_len, h_kv, _ = k.shape
+    if v.shape != k.shape:
+        raise ValueError(f"v {tuple(v.shape)} must have k's shape {tuple(k.shape)}")
+    if k.shape[0] != b or k.shape[-1] != head_dim:
+        raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
+    if head_dim not in (64, 128):
+        raise ValueError(f"head_dim {head_dim} not supported (64 or 128)")
+    if h_kv == 0 or h_qo % h_kv != 0:
+        raise ValueError(f"num_qo_heads {h_qo} must be a multiple of num_kv_heads {h_kv}")
+    nq = (qo_len + BLOCK_M - 1) // BLOCK_M
+    nk = (kv_len + BLOCK_N - 1) // BLOCK_N
+    if tuple(q_scale.shape) != (b, h_qo, nq) or tuple(k_scale.shape) != (b, h_kv, nk):
+        raise ValueError(
+            f"q_scale/k_scale must have shapes {(b, h_qo, nq)} / {(b, h_kv, nk)} (blocks of {BLOCK_M} / {BLOCK_N}), "
+            f"got {tuple(q_scale.shape)} / {tuple(k_scale.shape)}")
+    if q_scale.dtype != torch.float32 or k_scale.dtype != torch.float32:
+        raise TypeError("q_scale and k_scale must be float32")
+    q = q if rows_aligned(q) else q.contiguous()
+    k = k if rows_aligned(k) else k.contiguous()
+    v = v if rows_aligned(v) else v.contiguous()
+    q_scale = q_scale.contiguous()
+    k_scale = k_scale.contiguous()
+
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        o = torch.empty(q.shape, dtype=output_dtype, device=q.device)
+        if return_lse:
+            lse = torch.empty([b, h_qo, qo_len], dtype=torch.float32, device=q.device)
+        else:
+            lse = torch.empty([0], dtype=torch.float32, device="cpu")
+        if b == 0 or h_qo == 0 or qo_len == 0:
+            return o, lse
+        if kv_len == 0:  # no key: the reference's loop body never runs -> o = 0, lse = -inf
+            o.zero_()
+            if return_lse:
+                lse.fill_(float("-inf"))
+            return o, lse
+
+        p = _lib.AttnParams()
+        p.q, p.k, p.v, p.out = tensor_desc(q, hnd), tensor_desc(k, hnd), tensor_desc(v, hnd), tensor_desc(o, hnd)
+        p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
+        p.lse = lse.data_ptr() if return_lse else None
+        p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
+        p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
+        p.v_dtype, p.out_dtype = DTYPE_CODE[v.dtype], DTYPE_CODE[output_dtype]
+        p.causal = 1 if causal else 0
+        p.mask_kind = _lib.MASK_NONE
+        mask_keepalive = None
+        if attn_mask is not None:
+            require_gpu(attn_mask, "attn_mask")
+            m = attn_mask
+            if m.dtype == torch.bool:
+                p.mask_kind = _lib.MASK_BOOL
+            else:
+                p.mask_kind = _lib.MASK_F32
+                if m.dtype != torch.float32:
+                    m = m.float()
+            m = m.expand(b, h_qo, qo_len, kv_len)
+            mask_keepalive = m
+            p.mask = m.data_ptr()
+            p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = m.stride()
+        _lib.check(lib.sage_attn_fwd(ctypes.byref(p), current_stream_ptr(q.device)), "sage_attn_fwd")
+        del mask_keepalive
+    return o, lse

@@ -1,0 +1,140 @@
+"""``per_block_int8``: per-block INT8 quantization of Q and K on MI355X.
+
+Host side of FlagAttention's src/flag_attn/sage_attention/quant_per_block.py:49-101 with the
+same signature, defaults, outputs and errors.  The optional ``k - km`` smoothing (:53-54) is
+fused into the quantization kernel instead of running as a separate elementwise pass.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .. import _lib
+from ._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, tensor_desc
+
+_LOG2E = 1.44269504  # literal of quant_per_block.py:87
+
+
+def _f32(x: float) -> float:
+    return ctypes.c_float(x).value
+
+
+def k_mean(k: torch.Tensor, tensor_layout: str = "HND") -> torch.Tensor:
+    """Mean of K over the sequence axis in K's dtype, shape ``[B,H,1,D]`` (HND) / ``[B,1,H,D]``
+    (NHD), computed on the GPU in a fixed fp32 order (64-row chunks added row by row, chunk
+    partials added in order, one IEEE divide by N, one rounding) so that the result does not
+    depend on launch geometry.  This is what ``per_block_int8(..., smooth_k=True)`` passes as
+    ``km``; the reference leaves the mean to its caller (quant_per_block.py:49)."""
+    if tensor_layout not in ("HND", "NHD"):
+        raise ValueError(f"Unknown tensor layout: {tensor_layout}")
+    require_gpu(k, "k")
+    if k.dim() != 4:
+        raise ValueError(f"k must be 4-D, got shape {tuple(k.shape)}")
+    if k.dtype not in DTYPE_CODE:
+        raise TypeError(f"k dtype {k.dtype} not supported (float16, bfloat16, float32)")
+    hnd = tensor_layout == "HND"
+    if not rows_aligned(k):
+        k = k.contiguous()
+    if hnd:
+        b, h, n, d = k.shape
+    else:
+        b, n, h, d = k.shape
+    if n == 0:
+        raise ValueError("k_mean of an empty sequence")
+    lib = _lib.load()
+    with torch.cuda.device(k.device):
+        out = torch.empty((b, h, d), dtype=k.dtype, device=k.device)
+        ws = torch.empty(max(1, lib.sage_k_mean_workspace_bytes(b, h, n, d) // 4), dtype=torch.float32,
+                         device=k.device)
+        desc = tensor_desc(k, hnd)
+        _lib.check(lib.sage_k_mean(ctypes.byref(desc), DTYPE_CODE[k.dtype], out.data_ptr(), DTYPE_CODE[k.dtype],
+                                   b, h, n, d, ws.data_ptr(), current_stream_ptr(k.device)), "sage_k_mean")
+    return out.view(b, h, 1, d) if hnd else out.view(b, 1, h, d)
+
+
+def _prep_input(x: torch.Tensor, name: str) -> torch.Tensor:
+    require_gpu(x, name)
+    if x.dim() != 4:
+        raise ValueError(f"{name} must be 4-D, got shape {tuple(x.shape)}")
+    if x.dtype not in DTYPE_CODE:
+        raise TypeError(f"{name} dtype {x.dtype} not supported (float16, bfloat16, float32)")
+    return x if rows_aligned(x) else x.contiguous()
+
+
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", *, smooth_k=False):
+    """Returns ``(q_int8, q_scale, k_int8, k_scale)`` exactly as the reference does:
+    int8 tensors shaped like ``q`` / ``k`` and fp32 scales ``[B, Hq, ceil(M/BLKQ)]`` /
+    ``[B, Hkv, ceil(N/BLKK)]`` on ``q.device``.  Q is scaled by ``sm_scale * 1.44269504``
+    (default ``head_dim ** -0.5``) before quantization, K by nothing; ``km`` (any tensor
+    broadcastable to ``k``) is subtracted from K first with torch's rounding.
+
+    ``smooth_k=True`` (keyword only, not in the reference) computes ``km = k_mean(k)`` when no
+    ``km`` is given.
+    """
+    if tensor_layout not in ("HND", "NHD"):
+        raise ValueError(f"Unknown tensor layout: {tensor_layout}")
+    hnd = tensor_layout == "HND"
+    q = _prep_input(q, "q")
+    k = _prep_input(k, "k")
+    if hnd:
+        b, h_qo, qo_len, head_dim = q.shape
+        _, h_kv, kv_len, _ = k.shape
+    else:
+        b, qo_len, h_qo, head_dim = q.shape
+        _, kv_len, h_kv, _ = k.shape
+    if k.shape[0] != b or k.shape[-1] != head_dim:
+        raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
+    if k.device != q.device:
+        raise ValueError("q and k must be on the same device")
+    if km is None and smooth_k:
+        km = k_mean(k, tensor_layout)
+    if sm_scale is None:
+        sm_scale = head_dim ** -0.5
+    BLKQ, BLKK = int(BLKQ), int(BLKK)
+    if BLKQ <= 0 or BLKK <= 0:
+        raise ValueError("BLKQ and BLKK must be positive")
+
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        q_int8 = torch.empty(q.shape, dtype=torch.int8, device=q.device)
+        k_int8 = torch.empty(k.shape, dtype=torch.int8, device=k.device)
+        q_scale = torch.empty((b, h_qo, (qo_len + BLKQ - 1) // BLKQ), device=q.device, dtype=torch.float32)
+        k_scale = torch.empty((b, h_kv, (kv_len + BLKK - 1) // BLKK), device=q.device, dtype=torch.float32)
+
+        p = _lib.QuantParams()
+        p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
+        p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
+        p.blkq, p.blkk = BLKQ, BLKK
+        p.q_mul = _f32(sm_scale * _LOG2E)
+        p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
+        p.q_int8 = tensor_desc(q_int8, hnd)
+        p.k_int8 = tensor_desc(k_int8, hnd)
+        p.km = _lib.SageTensor(None, 0, 0, 0)
+        p.km_dtype = p.diff_dtype = _lib.SAGE_F32
+        km_keepalive = None
+        if km is not None:
+            require_gpu(km, "km")
+            if km.dtype not in DTYPE_CODE:
+                raise TypeError(f"km dtype {km.dtype} not supported (float16, bfloat16, float32)")
+            kme = km.expand(k.shape)
+            if not rows_aligned(kme):
+                kme = kme.contiguous()
+            km_keepalive = kme
+            p.km = tensor_desc(kme, hnd)
+            p.km_dtype = DTYPE_CODE[km.dtype]
+            p.diff_dtype = DTYPE_CODE[torch.result_type(k, km)]
+        stream = current_stream_ptr(q.device)
+        if q.dtype == k.dtype:
+            p.in_dtype = DTYPE_CODE[q.dtype]
+            p.q = tensor_desc(q, hnd)
+            p.k = tensor_desc(k, hnd)
+            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
+        else:
+            null = _lib.SageTensor(None, 0, 0, 0)
+            p.in_dtype, p.q, p.k = DTYPE_CODE[q.dtype], tensor_desc(q, hnd), null
+            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
+            p.in_dtype, p.q, p.k = DTYPE_CODE[k.dtype], null, tensor_desc(k, hnd)
+            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
+        del km_keepalive
+    return q_int8, q_scale, k_int8, k_scale

@@ -1,0 +1,117 @@
+/*
+ * C ABI of libsage_attention_hip.so: FlagAttention's SageAttention path on MI355X (gfx950).
+ *
+ * Plain pointers, sizes and strides only; no framework types.  All pointers are device
+ * pointers on the current HIP device unless stated otherwise; strides are in ELEMENTS and the
+ * innermost (head_dim) stride must be 1.  Tensors are described in the logical order
+ * (batch, head, sequence, head_dim); the reference's "HND" / "NHD" layouts differ only in
+ * which physical stride is passed as stride_h / stride_n.
+ *
+ * Every entry point enqueues work on `stream` (a hipStream_t passed as void*) and returns
+ * without synchronising.  Nothing is allocated or freed; outputs and the K-mean workspace are
+ * owned by the caller.  Return value: 0 on success, a negative SAGE_E_* code on a rejected call
+ * (nothing was launched); sage_hip_last_error() then returns a message for the calling thread.
+ */
+#ifndef SAGE_ATTENTION_HIP_H
+#define SAGE_ATTENTION_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum sage_dtype { SAGE_F16 = 0, SAGE_BF16 = 1, SAGE_F32 = 2 };
+enum sage_mask_kind { SAGE_MASK_NONE = 0, SAGE_MASK_BOOL = 1, SAGE_MASK_F32 = 2 };
+enum sage_status {
+    SAGE_OK = 0,
+    SAGE_E_INVALID = -1,     /* bad argument (shape, dtype, stride, null pointer) */
+    SAGE_E_UNSUPPORTED = -2, /* valid for the reference but not built here (e.g. head_dim) */
+    SAGE_E_LAUNCH = -3       /* the HIP runtime refused the launch */
+};
+
+/* A [B, H, L, D] tensor seen through strides (elements). */
+typedef struct sage_tensor {
+    void* ptr;
+    int64_t stride_b, stride_h, stride_n;
+} sage_tensor;
+
+/*
+ * Replaces the host function per_block_int8 and its two launches of
+ * quant_per_block_int8_kernel (src/flag_attn/sage_attention/quant_per_block.py:49-101, kernel
+ * :20-46), with the `k - km` pass (:53-54) fused into the K launch.
+ *
+ *   q, k         inputs, dtype in_dtype (SAGE_F16 / SAGE_BF16 / SAGE_F32)
+ *   km           optional (ptr == NULL: none) K mean, dtype km_dtype, broadcast through its own
+ *                strides (0 = broadcast); k - km is rounded once to diff_dtype exactly as the
+ *                torch subtraction it replaces (the promoted dtype of k and km)
+ *   q_int8,k_int8  outputs, int8, own strides
+ *   q_scale      [B, Hq, ceil(M/blkq)] fp32 contiguous;  k_scale [B, Hkv, ceil(N/blkk)]
+ *   q_mul        fp32 factor applied to Q before quantization (the reference passes
+ *                sm_scale * 1.44269504 rounded to fp32); a value of exactly 1.0f multiplies nothing
+ *   blkq, blkk   rows per quantization block (the attention kernel needs 128 / 64)
+ * Either of q.ptr / k.ptr may be NULL to quantize only the other tensor.
+ */
+typedef struct sage_quant_params {
+    sage_tensor q, k, km, q_int8, k_int8;
+    float* q_scale;
+    float* k_scale;
+    int64_t batch, heads_q, heads_kv, qo_len, kv_len, head_dim;
+    int32_t in_dtype, km_dtype, diff_dtype;
+    int32_t blkq, blkk;
+    float q_mul;
+} sage_quant_params;
+
+int sage_per_block_int8(const sage_quant_params* p, void* stream);
+
+/*
+ * Replaces the host function forward and its launch of _attn_fwd / _attn_fwd_inner
+ * (src/flag_attn/sage_attention/attn_qk_int8_per_block.py:129-191, kernels :20-127).
+ *
+ *   q, k         int8 (per_block_int8 outputs), v: v_dtype (SAGE_F16 / SAGE_BF16)
+ *   q_scale      [B, Hq, ceil(M/128)] fp32 contiguous;  k_scale [B, Hkv, ceil(N/64)]
+ *   out          out_dtype (SAGE_F16 / SAGE_BF16 / SAGE_F32), own strides
+ *   lse          optional [B, Hq, M] fp32 contiguous, base-2 log-sum-exp (:124-127); NULL = none
+ *   mask         optional [B, Hq, M, N] through 4 strides (elements, 0 = broadcast);
+ *                SAGE_MASK_BOOL: 1 byte per element, non-zero = keep (:33-36,48);
+ *                SAGE_MASK_F32: additive (:38,50)
+ *   causal       non-zero adds the bottom-right aligned causal mask n <= m + (N - M), handled
+ *                like a bool mask (tiles that are entirely masked are skipped)
+ * head_dim must be 64 or 128; heads_q must be a multiple of heads_kv.
+ */
+typedef struct sage_attn_params {
+    sage_tensor q, k, v, out;
+    const float* q_scale;
+    const float* k_scale;
+    float* lse;
+    const void* mask;
+    int64_t mask_stride_b, mask_stride_h, mask_stride_m, mask_stride_n;
+    int64_t batch, heads_q, heads_kv, qo_len, kv_len, head_dim;
+    int32_t v_dtype, out_dtype, mask_kind, causal;
+} sage_attn_params;
+
+int sage_attn_fwd(const sage_attn_params* p, void* stream);
+
+/*
+ * Mean of K over the sequence axis in a fixed fp32 order, for callers that want the library
+ * to produce the `km` argument of per_block_int8 (the reference leaves km to its caller,
+ * quant_per_block.py:49,53-54, so this entry point has no reference counterpart).
+ * Order: 64-row chunks summed row by row from 0.0f; chunk partials summed in order from 0.0f;
+ * total / (float)N; one rounding to out_dtype.  km_out: [B, Hkv, D] contiguous.
+ * workspace: at least sage_k_mean_workspace_bytes(...) bytes of device memory, 16-byte aligned.
+ */
+int64_t sage_k_mean_workspace_bytes(int64_t batch, int64_t heads_kv, int64_t kv_len, int64_t head_dim);
+int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out_dtype, int64_t batch,
+                int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* workspace, void* stream);
+
+/* Message describing the last non-zero status returned on this thread ("" if none). */
+const char* sage_hip_last_error(void);
+
+/* ABI version of this header; bumped when a struct layout changes. */
+int sage_hip_abi_version(void);
+#define SAGE_HIP_ABI_VERSION 1
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAGE_ATTENTION_HIP_H */

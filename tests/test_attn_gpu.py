@@ -1,0 +1,270 @@
+"""GPU parity of forward / sage_attention.
+
+Gate (north star): cosine >= 0.9995 and max-abs <= 2e-2 against the dequantized fp32 oracle on the
+same int8 inputs; the reference's own test tolerance atol = rtol = 2e-2 on output and LSE
+(tests/flag_attn/test_sage_attention.py:104-105,156-157) is asserted too.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import c_oracle as C
+from oracle import sage_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+COS_MIN = 0.9995
+MAX_ABS = 2e-2
+
+
+def _gate(actual, expected, what=""):
+    cos, rel, max_abs = O.accuracy_metrics(actual.float().cpu(), expected.float().cpu())
+    assert cos >= COS_MIN, f"{what}: cosine {cos}"
+    assert max_abs <= MAX_ABS, f"{what}: max-abs {max_abs}"
+    return cos, rel, max_abs
+
+
+def _quantized(seed, b, hq, hkv, m, n, d, dtype, layout="HND", k_offset=0.0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, hq, m, d, generator=g).to(dtype)
+    k = (torch.randn(b, hkv, n, d, generator=g) + k_offset).to(dtype)
+    v = torch.randn(b, hkv, n, d, generator=g).to(dtype)
+    if layout == "NHD":
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    q8, qs, k8, ks = O.per_block_int8(q, k, tensor_layout=layout)
+    return q8, qs, k8, ks, v
+
+
+def _run(dev, q8, qs, k8, ks, v, **kw):
+    from flag_attn import sage_attention as sa
+
+    o, lse = sa.sage_attention(q8.to(dev), k8.to(dev), v.to(dev), qs.to(dev), ks.to(dev), **kw)
+    torch.cuda.synchronize()
+    return o, lse
+
+
+@pytest.mark.parametrize("tensor_layout", ["HND", "NHD"])
+@pytest.mark.parametrize("num_kv_heads", [1, 2])
+def test_forward_matches_dequantized_reference(tensor_layout, num_kv_heads, gpu_device):
+    q8, qs, k8, ks, v = _quantized(2026, 1, 2, num_kv_heads, 128, 128, 64, torch.float16, tensor_layout)
+    actual, actual_lse = _run(gpu_device, q8, qs, k8, ks, v, tensor_layout=tensor_layout, return_lse=True)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, tensor_layout)
+    assert actual.dtype == torch.float16 and actual.shape == q8.shape
+    torch.testing.assert_close(actual.float().cpu(), expected, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(actual_lse.cpu(), expected_lse, atol=2e-2, rtol=2e-2)
+    _gate(actual, expected)
+
+
+def test_forward_rejects_non_positive_maxnreg(gpu_device):
+    from flag_attn import sage_attention as sa
+
+    q = torch.zeros((1, 1, 128, 64), device=gpu_device, dtype=torch.int8)
+    v = torch.zeros(q.shape, device=gpu_device, dtype=torch.float16)
+    q_scale = torch.ones((1, 1, 1), device=gpu_device)
+    k_scale = torch.ones((1, 1, 2), device=gpu_device)
+    with pytest.raises(ValueError, match="maxnreg must be positive"):
+        sa.sage_attention(q, q, v, q_scale, k_scale, maxnreg=0)
+    o, lse = sa.sage_attention(q, q, v, q_scale, k_scale, maxnreg=128)
+    assert lse.device.type == "cpu" and lse.numel() == 0 and lse.dtype == torch.float32
+    with pytest.raises(ValueError, match="tensor_layout XYZ not supported"):
+        sa.forward(q, q, v, q_scale, k_scale, tensor_layout="XYZ")
+
+
+@pytest.mark.parametrize("mask_kind", ["bool", "additive"])
+@pytest.mark.parametrize("kv_len", [70, 257])
+def test_forward_supports_masks_and_partial_blocks(mask_kind, kv_len, gpu_device):
+    q8, qs, k8, ks, v = _quantized(7, 1, 1, 1, 129, kv_len, 128, torch.float16)
+    if mask_kind == "bool":
+        attn_mask = torch.ones((1, 1, 129, kv_len), dtype=torch.bool)
+        attn_mask[..., ::3] = False
+    else:
+        attn_mask = torch.zeros((1, 1, 129, kv_len), dtype=torch.float32)
+        attn_mask[..., ::3] = -2.0
+    actual, actual_lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=attn_mask.to(gpu_device), return_lse=True)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, "HND", attn_mask)
+    torch.testing.assert_close(actual.float().cpu(), expected, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(actual_lse.cpu(), expected_lse, atol=2e-2, rtol=2e-2)
+    _gate(actual, expected)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("vdtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,n", [(128, 64), (1, 1), (200, 333), (512, 512), (77, 1000)])
+def test_shapes_dtypes(d, vdtype, m, n, gpu_device):
+    q8, qs, k8, ks, v = _quantized(11, 2, 4, 2, m, n, d, vdtype)
+    for out_dtype in (torch.float16, torch.bfloat16, torch.float32):
+        actual, lse = _run(gpu_device, q8, qs, k8, ks, v, output_dtype=out_dtype, return_lse=True)
+        assert actual.dtype == out_dtype
+        expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks)
+        _gate(actual, expected, f"{out_dtype}")
+        torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("m,n", [(256, 256), (129, 257), (300, 100), (64, 640), (1, 130)])
+def test_causal(layout, m, n, gpu_device):
+    q8, qs, k8, ks, v = _quantized(3, 1, 2, 1, m, n, 128, torch.bfloat16, layout)
+    actual, lse = _run(gpu_device, q8, qs, k8, ks, v, tensor_layout=layout, causal=True, return_lse=True)
+    # kernel-faithful oracle: rows with no visible key are defined by the -1e6 / tile-skip rules
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, layout, causal=True)
+    _gate(actual, expected)
+    fin = torch.isfinite(expected_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    torch.testing.assert_close(lse.cpu()[fin], expected_lse[fin], atol=2e-2, rtol=2e-2)
+    if n >= m:  # every row sees a key: the closed form applies as well
+        ref, ref_lse = O.attention_dequant(q8, k8, v, qs, ks, layout, causal=True)
+        _gate(actual, ref)
+        torch.testing.assert_close(lse.cpu(), ref_lse, atol=2e-3, rtol=1e-4)
+
+
+def test_mask_edge_semantics(gpu_device):
+    q8, qs, k8, ks, v = _quantized(5, 1, 2, 2, 130, 200, 64, torch.float16)
+    # all-False mask: every tile skipped -> o = 0, lse = -inf
+    mask = torch.zeros(1, 2, 130, 200, dtype=torch.bool)
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask.to(gpu_device), return_lse=True)
+    assert float(o.abs().max()) == 0.0 and bool((lse == float("-inf")).all())
+    # only the middle tile has visible keys, and row 7 sees none of them: -1e6 semantics (no NaN)
+    mask[..., 64:128] = True
+    mask[:, :, 7, :] = False
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask.to(gpu_device), return_lse=True)
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, attn_mask=mask)
+    assert bool(torch.isfinite(o).all())
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=1.0, rtol=1e-5)  # lse of a masked row is ~ -1e6
+    # broadcast mask [1,1,M,N] over batch and heads, bool
+    bm = torch.rand(1, 1, 130, 200, generator=torch.Generator().manual_seed(1)) > 0.3
+    bm[..., 0] = True
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=bm.to(gpu_device), return_lse=True)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, attn_mask=bm)
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
+
+
+def test_uniform_v_and_zero_scale_block(gpu_device):
+    q8, qs, k8, ks, v = _quantized(8, 1, 1, 1, 256, 256, 128, torch.bfloat16)
+    vu = v[:, :, :1].expand_as(v).contiguous()
+    o, _ = _run(gpu_device, q8, qs, k8, ks, vu, output_dtype=torch.float32)
+    torch.testing.assert_close(o.cpu(), vu[:, :, :1].float().expand_as(o), atol=4e-3, rtol=4e-3)
+    ks2 = ks.clone()
+    ks2[..., 1] = 0.0  # an all-zero K block quantizes to scale 0: its scores are exactly 0
+    o, lse = _run(gpu_device, q8, qs, k8, ks2, v, return_lse=True)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks2)
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
+
+
+def _gpu_dequant_reference(q8, k8, v, qs, ks, heads, causal=False):
+    """fp32 softmax attention of the dequantized operands for a few (batch, head) pairs, on the GPU
+    (the same closed form as the oracle's attention_dequant; used where the CPU would take minutes)."""
+    outs = []
+    for b, h in heads:
+        hk = h // (q8.shape[1] // k8.shape[1])
+        q = q8[b, h].float() * qs[b, h].repeat_interleave(128)[: q8.shape[2], None]
+        k = k8[b, hk].float() * ks[b, hk].repeat_interleave(64)[: k8.shape[2], None]
+        s = (q @ k.T) * math.log(2.0)
+        if causal:
+            m, n = s.shape
+            s = s.masked_fill(~(torch.arange(n, device=s.device)[None] <= torch.arange(m, device=s.device)[:, None] + (n - m)),
+                              float("-inf"))
+        outs.append(torch.softmax(s, dim=-1) @ v[b, hk].float())
+    return torch.stack(outs)
+
+
+def test_north_star_config_full_size(gpu_device):
+    """B4 H32 N4096 D128 bf16 HND non-causal, K smoothing on: CPU oracle on two heads, GPU fp32
+    closed form on eight, benchmark-style gate against SDPA on the unquantized inputs."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(4, 32, 4096, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    qd, kd, vd = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
+    q8, qs, k8, ks = sa.per_block_int8(qd, kd, smooth_k=True)
+    o, lse = sa.sage_attention(q8, k8, vd, qs, ks, output_dtype=torch.bfloat16, return_lse=True)
+    torch.cuda.synchronize()
+    heads = [(0, 0), (3, 31)]
+    for b, h in heads:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        exp, exp_lse = C.attention_blockwise(q8[sl].cpu(), k8[sl].cpu(), v[sl], qs[sl].cpu(), ks[sl].cpu())
+        _gate(o[sl], exp, f"head {b},{h}")
+        torch.testing.assert_close(lse[sl].cpu(), exp_lse, atol=2e-3, rtol=1e-4)
+    heads = [(b, h) for b in range(4) for h in (5, 20)]
+    ref = _gpu_dequant_reference(q8, k8, vd, qs, ks, heads)
+    got = torch.stack([o[b, h] for b, h in heads])
+    _gate(got, ref, "gpu closed form")
+    base = torch.nn.functional.scaled_dot_product_attention(qd[:1], kd[:1], vd[:1])
+    cos, rel, _ = O.accuracy_metrics(o[:1].cpu(), base.cpu())
+    assert cos >= 0.99 and rel <= 0.05  # benchmark/test_sage_attention_benchmark.py:174-177
+
+
+def test_causal_nhd_config_shape(gpu_device):
+    """B2 H32 N8192 D128 NHD bf16 causal, K = N(0,1) + per-channel offset N(0,4) (batch cut to 1)."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(42)
+    b, n, h, d = 1, 8192, 32, 128
+    q = torch.randn(b, n, h, d, generator=g).to(torch.bfloat16)
+    k = (torch.randn(b, n, h, d, generator=g) + 2.0 * torch.randn(1, 1, h, d, generator=g)).to(torch.bfloat16)
+    v = torch.randn(b, n, h, d, generator=g).to(torch.bfloat16)
+    qd, kd, vd = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
+    q8, qs, k8, ks = sa.per_block_int8(qd, kd, tensor_layout="NHD", smooth_k=True)
+    o, _ = sa.sage_attention(q8, k8, vd, qs, ks, tensor_layout="NHD", output_dtype=torch.bfloat16, causal=True)
+    heads = [(0, 0), (0, 17), (0, 31)]
+    ref = _gpu_dequant_reference(q8.transpose(1, 2), k8.transpose(1, 2), vd.transpose(1, 2), qs, ks, heads, causal=True)
+    got = torch.stack([o[bb, :, hh] for bb, hh in heads])
+    _gate(got, ref)
+    base = torch.nn.functional.scaled_dot_product_attention(
+        qd.transpose(1, 2)[:, :4], kd.transpose(1, 2)[:, :4], vd.transpose(1, 2)[:, :4], is_causal=True)
+    cos, rel, _ = O.accuracy_metrics(o.transpose(1, 2)[:, :4].cpu(), base.cpu())
+    assert cos >= 0.99 and rel <= 0.05
+
+
+def test_outlier_d64_config_shape(gpu_device):
+    """B8 H16 N2048 D64 fp16, 1% outlier channels x20 in Q and K, V ~ U(-1,1) (batch cut to 2)."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(42)
+    b, h, n, d = 2, 16, 2048, 64
+    q = torch.randn(b, h, n, d, generator=g)
+    k = torch.randn(b, h, n, d, generator=g)
+    idx = torch.randperm(h * d, generator=g)[:10]
+    for t in (q, k):
+        t.permute(0, 2, 1, 3).reshape(b, n, h * d)[..., idx] *= 20
+    v = torch.rand(b, h, n, d, generator=g) * 2 - 1
+    q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
+    q8, qs, k8, ks = sa.per_block_int8(q.to(gpu_device), k.to(gpu_device))
+    o, lse = sa.sage_attention(q8, k8, v.to(gpu_device), qs, ks, return_lse=True)
+    exp, exp_lse = C.attention_blockwise(q8[:1, :4].cpu(), k8[:1, :4].cpu(), v[:1, :4], qs[:1, :4].cpu(), ks[:1, :4].cpu())
+    _gate(o[:1, :4], exp)
+    torch.testing.assert_close(lse[:1, :4].cpu(), exp_lse, atol=2e-3, rtol=1e-4)
+    heads = [(bb, hh) for bb in range(b) for hh in (3, 9, 15)]
+    ref = _gpu_dequant_reference(q8, k8, v.to(gpu_device), qs, ks, heads)
+    _gate(torch.stack([o[bb, hh] for bb, hh in heads]), ref)
+
+
+def test_long_sequence_config_shape(gpu_device):
+    """B1 H24 N32768 D128 bf16 non-causal, K smoothing on (heads cut to 4)."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(1, 4, 32768, 128, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
+    q8, qs, k8, ks = sa.per_block_int8(q, k, smooth_k=True)
+    o, _ = sa.sage_attention(q8, k8, v, qs, ks, output_dtype=torch.bfloat16)
+    ref = _gpu_dequant_reference(q8, k8, v, qs, ks, [(0, 1)])
+    _gate(o[0, 1][None], ref)
+
+
+def test_sageattn_wrapper_lse(gpu_device):
+    from flag_attn.sage_attention import sageattn
+
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(1, 4, 300, 128, generator=g).to(torch.bfloat16).to(gpu_device)
+    k = (torch.randn(1, 2, 500, 128, generator=g) + 1.5).to(torch.bfloat16).to(gpu_device)
+    v = torch.randn(1, 2, 500, 128, generator=g).to(torch.bfloat16).to(gpu_device)
+    o, lse = sageattn(q, k, v, return_lse=True)
+    kk, vv = k.repeat_interleave(2, 1).float(), v.repeat_interleave(2, 1).float()
+    s = (q.float() @ kk.transpose(-1, -2)) * 128 ** -0.5
+    ref = torch.softmax(s, -1) @ vv
+    cos, rel, _ = O.accuracy_metrics(o.cpu(), ref.cpu())
+    assert cos >= 0.999 and rel <= 0.05
+    torch.testing.assert_close(lse, torch.logsumexp(s, -1), atol=5e-2, rtol=1e-3)

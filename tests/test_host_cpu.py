@@ -1,0 +1,87 @@
+"""CPU-only checks of the host side: the C-ABI library loads and exports every symbol the header
+declares, structs match the header, argument errors surface before any GPU work."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sage_attention_hip.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sage_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from flagattention_amd import _lib
+
+    lib = _lib.load()
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.sage_hip_abi_version() == _lib.ABI_VERSION
+    assert lib.sage_hip_last_error() == b"" or isinstance(lib.sage_hip_last_error(), bytes)
+
+
+def test_struct_layouts_match_header():
+    from flagattention_amd import _lib
+
+    # sizes follow from the header's field lists: 4x8; 5*32 + 2*8 + 6*8 + 5*4 + 4 (+pad to 8)
+    assert ctypes.sizeof(_lib.SageTensor) == 32
+    assert ctypes.sizeof(_lib.QuantParams) == 5 * 32 + 2 * 8 + 6 * 8 + 6 * 4
+    assert ctypes.sizeof(_lib.AttnParams) == 4 * 32 + 4 * 8 + 4 * 8 + 6 * 8 + 4 * 4
+
+
+def test_validation_without_gpu_work():
+    """Rejected calls return before any launch, so they are safe on a machine with no GPU."""
+    from flagattention_amd import _lib
+
+    lib = _lib.load()
+    assert lib.sage_per_block_int8(None, None) == -1
+    assert b"null params" in lib.sage_hip_last_error()
+    p = _lib.AttnParams()
+    assert lib.sage_attn_fwd(ctypes.byref(p), None) == -1
+    p.q.ptr = p.k.ptr = p.v.ptr = p.out.ptr = 4096
+    p.q_scale = p.k_scale = 4096
+    p.head_dim = 96
+    assert lib.sage_attn_fwd(ctypes.byref(p), None) == -2
+    assert b"head_dim 96" in lib.sage_hip_last_error()
+    p.head_dim, p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len = 128, 1, 3, 2, 8, 8
+    assert lib.sage_attn_fwd(ctypes.byref(p), None) == -1
+    assert b"multiple of heads_kv" in lib.sage_hip_last_error()
+    assert lib.sage_k_mean_workspace_bytes(2, 3, 130, 64) == 2 * 3 * 3 * 64 * 4
+
+
+def test_python_api_errors_on_cpu():
+    from flag_attn import sage_attention as sa
+
+    assert sa.sage_attention is sa.forward
+    q = torch.zeros(1, 1, 128, 64, dtype=torch.int8)
+    v = torch.zeros(1, 1, 128, 64, dtype=torch.float16)
+    s = torch.ones(1, 1, 1)
+    with pytest.raises(ValueError, match="maxnreg must be positive"):
+        sa.sage_attention(q, q, v, s, torch.ones(1, 1, 2), maxnreg=0)
+    with pytest.raises(ValueError, match="tensor_layout ABC not supported"):
+        sa.forward(q, q, v, s, s, tensor_layout="ABC")
+    with pytest.raises(ValueError, match="Unknown tensor layout: ABC"):
+        sa.per_block_int8(v, v, tensor_layout="ABC")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        sa.per_block_int8(v, v)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        sa.forward(q, q, v, s, torch.ones(1, 1, 2))
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "flagattention_amd")
+    for base in (pkg, os.path.join(ROOT, "flag_attn")):
+        for dirpath, _, files in os.walk(base):
+            for f in files:
+                if f.endswith((".py", ".hip", ".cpp", ".h")):
+                    text = open(os.path.join(dirpath, f)).read()
+                    assert "oracle" not in text.lower(), os.path.join(dirpath, f)

@@ -1,0 +1,150 @@
+"""GPU parity of per_block_int8 / k_mean against the CPU oracle: bit-exact int8 and scales."""
+import pytest
+import torch
+
+from golden_io import load_cases
+from oracle import c_oracle as C
+from oracle import sage_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+CASES = load_cases()
+
+
+def _gpu(t, dev):
+    return None if t is None else t.to(dev)
+
+
+def _assert_bit_exact(got, want):
+    for g, w, name in zip(got, want, ("q_int8", "q_scale", "k_int8", "k_scale")):
+        g = g.cpu()
+        assert g.dtype == w.dtype and g.shape == w.shape, name
+        if g.dtype == torch.float32:
+            assert torch.equal(g.view(torch.int32), w.view(torch.int32)), f"{name}: scale bits differ"
+        else:
+            nbad = int((g != w).sum())
+            assert nbad == 0, f"{name}: {nbad} of {g.numel()} int8 values differ"
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["name"] for c in CASES])
+def test_golden_vectors(case, gpu_device):
+    from flag_attn.sage_attention import per_block_int8
+
+    got = per_block_int8(_gpu(case["q"], gpu_device), _gpu(case["k"], gpu_device), km=_gpu(case["km"], gpu_device),
+                         **case["kw"])
+    assert got[1].device == got[0].device and got[3].device == got[0].device
+    _assert_bit_exact(got, (case["q_int8"], case["q_scale"], case["k_int8"], case["k_scale"]))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("with_km", [False, True])
+def test_random_vs_oracle(dtype, layout, with_km, gpu_device):
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(1234)
+    b, hq, hkv, m, n, d = 2, 4, 2, 333, 517, 128
+    q = torch.randn(b, hq, m, d, generator=g).to(dtype)
+    k = (torch.randn(b, hkv, n, d, generator=g) + torch.randn(1, hkv, 1, d, generator=g) * 2).to(dtype)
+    km = k.float().mean(dim=2, keepdim=True).to(dtype) if with_km else None
+    if layout == "NHD":
+        q, k = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+        km = km.transpose(1, 2).contiguous() if with_km else None
+    want = O.per_block_int8(q, k, km=km, tensor_layout=layout)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=_gpu(km, gpu_device), tensor_layout=layout)
+    _assert_bit_exact(got, want)
+
+
+@pytest.mark.parametrize("blkq,blkk,d", [(64, 32, 64), (32, 16, 128), (256, 128, 64), (128, 64, 96), (16, 16, 32)])
+def test_block_sizes_and_head_dims(blkq, blkk, d, gpu_device):
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(1, 3, 300, d, generator=g).to(torch.float16)
+    k = torch.randn(1, 3, 130, d, generator=g).to(torch.float16)
+    want = O.per_block_int8(q, k, BLKQ=blkq, BLKK=blkk, sm_scale=0.77)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), BLKQ=blkq, BLKK=blkk, sm_scale=0.77)
+    _assert_bit_exact(got, want)
+
+
+def test_strided_views_and_mixed_dtypes(gpu_device):
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(5)
+    big = torch.randn(2, 2, 200, 256, generator=g).to(torch.bfloat16)
+    q = big[..., :128]  # row stride 256, still 16-byte aligned rows
+    k = torch.randn(2, 2, 100, 128, generator=g).to(torch.float16)
+    km = k.float().mean(dim=2, keepdim=True)  # fp32 km against fp16 k
+    want = O.per_block_int8(q, k, km=km)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=km.to(gpu_device))
+    _assert_bit_exact(got, want)
+    odd = big[..., 1:129]  # rows not 16-byte aligned: the wrapper must copy
+    want = O.per_block_int8(odd, k)
+    got = per_block_int8(odd.to(gpu_device)[..., :], k.to(gpu_device))
+    _assert_bit_exact(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+def test_k_mean_bit_exact(dtype, layout, gpu_device):
+    from flag_attn.sage_attention import k_mean, per_block_int8
+
+    g = torch.Generator().manual_seed(9)
+    k = (torch.randn(2, 3, 1000, 128, generator=g) + torch.randn(1, 3, 1, 128, generator=g) * 2).to(dtype)
+    q = torch.randn(2, 3, 256, 128, generator=g).to(dtype)
+    if layout == "NHD":
+        k, q = k.transpose(1, 2).contiguous(), q.transpose(1, 2).contiguous()
+    want = C.k_mean_fixed_order(k, layout)
+    got = k_mean(k.to(gpu_device), layout)
+    assert got.shape == want.shape and got.dtype == want.dtype
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    want_q = O.per_block_int8(q, k, km=want, tensor_layout=layout)
+    got_q = per_block_int8(q.to(gpu_device), k.to(gpu_device), tensor_layout=layout, smooth_k=True)
+    _assert_bit_exact(got_q, want_q)
+
+
+def test_outlier_channels_config4_shape(gpu_device):
+    """B8 H16 N2048 D64 fp16 with 1% of (head, dim) channels x20: saturation only at +-127."""
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(42)
+    b, h, n, d = 2, 16, 2048, 64  # batch cut to 2 of 8: blocks are independent
+    q = torch.randn(b, h, n, d, generator=g)
+    k = torch.randn(b, h, n, d, generator=g)
+    idx = torch.randperm(h * d, generator=g)[:10]
+    for t in (q, k):
+        t.view(b, h, n, d).permute(0, 2, 1, 3).reshape(b, n, h * d)[..., idx] *= 20
+    q, k = q.to(torch.float16), k.to(torch.float16)
+    want = O.per_block_int8(q, k)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device))
+    _assert_bit_exact(got, want)
+    assert int(got[0].min()) >= -127 and int(got[2].min()) >= -127
+
+
+def test_north_star_shape_bit_exact(gpu_device):
+    """B4 H32 N4096 D128 bf16 HND with K smoothing, the benchmark configuration, at full size."""
+    from flag_attn.sage_attention import k_mean, per_block_int8
+
+    g = torch.Generator().manual_seed(42)
+    q = torch.randn(4, 32, 4096, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(4, 32, 4096, 128, generator=g).to(torch.bfloat16)
+    km = k_mean(k.to(gpu_device)).cpu()
+    assert torch.equal(km.view(torch.int16), C.k_mean_fixed_order(k).view(torch.int16))
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=km.to(gpu_device))
+    want = O.per_block_int8(q, k, km=km)
+    _assert_bit_exact(got, want)
+    # size-independent properties on the device result
+    q8, qs, k8, ks = got
+    assert int(q8.abs().amax()) == 127 and int(q8.min()) >= -127
+    assert bool((q8.view(4, 32, 32, 128 * 128).abs().amax(-1) == 127).all())
+    assert bool((k8.view(4, 32, 64, 64 * 128).abs().amax(-1) == 127).all())
+
+
+def test_errors(gpu_device):
+    from flag_attn.sage_attention import per_block_int8
+
+    q = torch.zeros(1, 1, 128, 64, device=gpu_device, dtype=torch.float16)
+    with pytest.raises(ValueError, match="Unknown tensor layout: XYZ"):
+        per_block_int8(q, q, tensor_layout="XYZ")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        per_block_int8(q.cpu(), q.cpu())
