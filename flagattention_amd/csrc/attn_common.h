@@ -1,0 +1,75 @@
+// Types shared by the attention kernels of libsage_attention_hip.so (gfx950).
+#pragma once
+#include "common.h"
+
+namespace sage {
+namespace attn {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kThreads = 256;
+constexpr int BM = 128;  // query rows per workgroup (= Q quantization block)
+constexpr int BN = 64;   // keys per step (= K quantization block)
+constexpr float kMasked = -1.0e6f;
+constexpr float kTau = 8.0f;  // log2 of the largest P tolerated before the running maximum is advanced
+
+enum { MODE_PLAIN = 0, MODE_CAUSAL = 1, MODE_MASK_BOOL = 2, MODE_MASK_F32 = 3 };
+
+struct AttnArgs {
+    const int8_t* q;
+    const int8_t* k;
+    const void* v;
+    void* out;
+    const float* q_scale;
+    const float* k_scale;
+    float* lse;
+    const void* mask;
+    int64_t qs_b, qs_h, qs_n;
+    int64_t ks_b, ks_h, ks_n;
+    int64_t vs_b, vs_h, vs_n;
+    int64_t os_b, os_h, os_n;
+    int64_t ms_b, ms_h, ms_m, ms_n;
+    int32_t Hq, Hkv, M, N, nq, nk, groups;
+    int32_t out_dt, causal;
+    int32_t total_wg;
+};
+
+template <typename VT> struct PV;
+template <> struct PV<__bf16> {
+    typedef bf16x8 vec;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    // acc + p[2c] + p[2c+1]
+    static __device__ __forceinline__ float dot2_ones(vec p, int c, float acc) {
+        typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+        const v2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+        const v2 pr = {p[2 * c], p[2 * c + 1]};
+        return __builtin_amdgcn_fdot2_f32_bf16(pr, ones, acc, false);
+    }
+};
+template <> struct PV<_Float16> {
+    typedef f16x8 vec;
+    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float dot2_ones(vec p, int c, float acc) {
+        typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+        const v2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+        const v2 pr = {p[2 * c], p[2 * c + 1]};
+        return __builtin_amdgcn_fdot2(pr, ones, acc, false);
+    }
+};
+
+
+// Launches the software-pipelined kernel for the common case (no mask tensor, kv_len a multiple
+// of 64, and qo_len <= kv_len when causal).  head_dim 64 / 128, V dtype fp16 / bf16.
+int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream);
+
+}  // namespace attn
+}  // namespace sage

@@ -20,57 +20,11 @@
 //   exactly the order the S^T accumulator layout dictates (see v_chunk()).
 //   K tiles (int8 [64][D]) and V tiles (16-bit, transposed to [D][64]) are double buffered in LDS;
 //   global loads for step j+1 are issued before the math of step j.
-#include "common.h"
+#include "attn_common.h"
 
 namespace sage {
+using namespace attn;
 namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-constexpr int kThreads = 256;
-constexpr int BM = 128;  // query rows per workgroup (= Q quantization block)
-constexpr int BN = 64;   // keys per step (= K quantization block)
-constexpr float kMasked = -1.0e6f;
-
-enum { MODE_PLAIN = 0, MODE_CAUSAL = 1, MODE_MASK_BOOL = 2, MODE_MASK_F32 = 3 };
-
-struct AttnArgs {
-    const int8_t* q;
-    const int8_t* k;
-    const void* v;
-    void* out;
-    const float* q_scale;
-    const float* k_scale;
-    float* lse;
-    const void* mask;
-    int64_t qs_b, qs_h, qs_n;
-    int64_t ks_b, ks_h, ks_n;
-    int64_t vs_b, vs_h, vs_n;
-    int64_t os_b, os_h, os_n;
-    int64_t ms_b, ms_h, ms_m, ms_n;
-    int32_t Hq, Hkv, M, N, nq, nk, groups;
-    int32_t out_dt, causal;
-    int32_t total_wg;
-};
-
-template <typename VT> struct PV;
-template <> struct PV<__bf16> {
-    typedef bf16x8 vec;
-    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct PV<_Float16> {
-    typedef f16x8 vec;
-    static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
 
 template <int D>
 struct Tile {
@@ -158,40 +112,56 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
     // ---- staging roles
     const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
     const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
-    int k_row[T::K_LOADS], k_lds[T::K_LOADS], k_goff[T::K_LOADS];
+    int k_row[T::K_LOADS], k_lds[T::K_LOADS], k_col[T::K_LOADS], k_off[T::K_LOADS];
 #pragma unroll
     for (int j = 0; j < T::K_LOADS; j++) {
         const int id = tid + kThreads * j;
         k_row[j] = id / T::K_CHUNKS_PER_ROW;
-        const int c = id % T::K_CHUNKS_PER_ROW;
-        k_lds[j] = k_row[j] * T::K_RS + 16 * c;
-        k_goff[j] = 16 * c;
+        k_col[j] = 16 * (id % T::K_CHUNKS_PER_ROW);
+        k_lds[j] = k_row[j] * T::K_RS + k_col[j];
+        k_off[j] = k_row[j] * (int)a.ks_n + k_col[j];  // byte offset inside a tile (host checks it fits 31 bits)
     }
     const bool v_worker = tid < T::V_ITEMS;
     const int v_dg = tid % (D / 8);  // group of 8 channels
     const int v_r = tid / (D / 8);   // run of 4 keys
-    int v_lds[8];
+    int v_lds[8], v_off[4];
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const int d = 8 * v_dg + e;
         v_lds[e] = T::K_BYTES + d * T::V_RS + ((v_chunk(v_r) ^ v_swz(d)) * 16) + v_halfchunk(v_r) * 8;
     }
+#pragma unroll
+    for (int i = 0; i < 4; i++) v_off[i] = (4 * v_r + i) * (int)a.vs_n + 8 * v_dg;  // element offset inside a tile
 
     v4i kreg[T::K_LOADS];
     uint4 vreg[4];
     auto load_tile = [&](int step) {
         const int n0 = step * BN;
+        const int8_t* kt = kg + (int64_t)n0 * a.ks_n;  // uniform tile bases, 32-bit per-lane offsets
+        const VT* vt = vg + (int64_t)n0 * a.vs_n;
+        if (n0 + BN <= a.N) {
 #pragma unroll
-        for (int j = 0; j < T::K_LOADS; j++) {
-            const int n = n0 + k_row[j];
-            kreg[j] = (n < a.N) ? *reinterpret_cast<const v4i*>(kg + (int64_t)n * a.ks_n + k_goff[j]) : v4i{0, 0, 0, 0};
-        }
-        if (v_worker) {
+            for (int j = 0; j < T::K_LOADS; j++) kreg[j] = *reinterpret_cast<const v4i*>(kt + k_off[j]);
+            if (v_worker) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int n = n0 + 4 * v_r + i;
-                vreg[i] = (n < a.N) ? *reinterpret_cast<const uint4*>(vg + (int64_t)n * a.vs_n + 8 * v_dg)
-                                    : make_uint4(0, 0, 0, 0);
+                for (int i = 0; i < 4; i++) vreg[i] = *reinterpret_cast<const uint4*>(vt + v_off[i]);
+            }
+        } else {
+            // last, partial tile: keys past N read as zeros (their scores get -1e6, their V rows weigh 0)
+            const int last = a.N - 1 - n0;
+#pragma unroll
+            for (int j = 0; j < T::K_LOADS; j++) {
+                const int r = min(k_row[j], last);
+                kreg[j] = *reinterpret_cast<const v4i*>(kt + (int64_t)r * a.ks_n + k_col[j]);
+                if (k_row[j] > last) kreg[j] = v4i{0, 0, 0, 0};
+            }
+            if (v_worker) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = min(4 * v_r + i, last);
+                    vreg[i] = *reinterpret_cast<const uint4*>(vt + (int64_t)r * a.vs_n + 8 * v_dg);
+                    if (4 * v_r + i > last) vreg[i] = make_uint4(0, 0, 0, 0);
+                }
             }
         }
     };
@@ -326,39 +296,44 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
                     }
                 rmax = xhalf_max(rmax);
             }
+            // The running maximum is only advanced (and O, l rescaled) when some row of this wave
+            // moved by more than kTau; otherwise exponentials are taken against the stale maximum
+            // (p <= 2^kTau, exact in the final o = O / l and lse = log2(l) + m).
             const float m_new = fmaxf(m_i, rmax);
-            const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-            float lsum = 0.0f;
+            if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+                l_i *= alpha;
+                m_i = m_new;
+#pragma unroll
+                for (int dt = 0; dt < T::DTILES; dt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+            }
             if (plain) {
 #pragma unroll
                 for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        s[kt][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], sc, -m_new));
-                        lsum += s[kt][i];
-                    }
+                    for (int i = 0; i < 16; i++) s[kt][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], sc, -m_i));
             } else {
 #pragma unroll
                 for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        s[kt][i] = __builtin_amdgcn_exp2f(s[kt][i] - m_new);
-                        lsum += s[kt][i];
-                    }
+                    for (int i = 0; i < 16; i++) s[kt][i] = __builtin_amdgcn_exp2f(s[kt][i] - m_i);
             }
-            l_i = l_i * alpha + lsum;
-            m_i = m_new;
-#pragma unroll
-            for (int dt = 0; dt < T::DTILES; dt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
 
-            // ---- P^T as the B operand: k-step t' of 16 keys takes S^T registers 8(t'&1) .. +7 of tile t'>>1
+            // ---- P^T as the B operand: k-step t' of 16 keys takes S^T registers 8(t'&1) .. +7 of tile t'>>1.
+            //      The row sum is taken over the rounded P (pairs through v_dot2), so that numerator and
+            //      denominator of o = O / l see the same weights.
             vec16 pf[4];
+            float lsum = 0.0f;
 #pragma unroll
-            for (int tp = 0; tp < 4; tp++)
+            for (int tp = 0; tp < 4; tp++) {
 #pragma unroll
                 for (int c = 0; c < 8; c++) pf[tp][c] = (VT)s[tp >> 1][8 * (tp & 1) + c];
+#pragma unroll
+                for (int c = 0; c < 4; c++) lsum = PVT::dot2_ones(pf[tp], c, lsum);
+            }
+            l_i += lsum;
 
             // ---- O^T += V^T . P^T
 #pragma unroll
@@ -433,11 +408,16 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     const int64_t total = p.batch * p.heads_q * a.nq;
     if (total > 0x7fffffffLL || p.qo_len > 0x7fffffffLL - BM || p.kv_len > 0x7fffffffLL - BN)
         return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: problem too large for 32-bit tile indices");
+    if (p.k.stride_n < 0 || p.v.stride_n < 0 || (int64_t)BN * p.k.stride_n >= (1LL << 30) ||
+        (int64_t)BN * p.v.stride_n >= (1LL << 29))
+        return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: k/v sequence stride out of range for 32-bit tile offsets");
     a.total_wg = (int)total;
     int mode = MODE_PLAIN;
     if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
     else if (p.mask_kind == SAGE_MASK_F32) mode = MODE_MASK_F32;
     else if (p.causal) mode = MODE_CAUSAL;
+    const bool fast = p.mask_kind == SAGE_MASK_NONE && (p.kv_len % BN) == 0 && (!p.causal || p.qo_len <= p.kv_len);
+    if (fast) return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
     if (p.head_dim == 128) {
         return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)
                                       : launch_mode<128, _Float16>(a, mode, stream);

@@ -1,0 +1,337 @@
+// Software-pipelined SageAttention forward for gfx950: the common case (no mask tensor, kv_len a
+// multiple of 64, causal only with qo_len <= kv_len).  Same arithmetic contract as the general
+// kernel in attn_fwd.hip (FlagAttention src/flag_attn/sage_attention/attn_qk_int8_per_block.py:
+// 20-127); what differs is how the work is laid out in time.
+//
+// Per workgroup: 8 waves x 32 query rows (two q_scale blocks, so that every K/V tile staged in LDS
+// serves 256 rows); per step: 64 keys.  Every wave computes the transposed
+// products S^T = K.Q^T (8 x v_mfma_i32_32x32x32_i8) and O^T += V^T.P^T (16 x v_mfma_f32_32x32x16)
+// so that a lane owns one query row and P never leaves registers.
+//
+// * V is staged in LDS as it lies in memory ([key][channel], rows padded by 64 bytes) and read
+//   with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel: exactly
+//   the A operand of the P.V MFMA, with no shuffling instructions.
+// * The loop is skewed by one step: while the exponentials of step j run on the VALU, the matrix
+//   core works on Q.K^T of step j+1 and then on P.V of step j, whose tail overlaps the row-max
+//   pass of the next iteration.  K of step j+2 and V of step j+1 are fetched from global memory
+//   into registers at the top of iteration j and stored to LDS at its end (one barrier per step).
+// * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
+//   rare steps where a row maximum jumps.
+#include "attn_common.h"
+
+namespace sage {
+namespace attn {
+namespace {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+
+constexpr int kFastThreads = 512;  // 8 waves
+constexpr int kFastRows = 256;     // query rows per workgroup
+
+template <int D>
+struct FT {
+    static constexpr int KSTEPS = D / 32;
+    static constexpr int DTILES = D / 32;
+    static constexpr int K_RS = D + 16;       // bytes per K row in LDS
+    static constexpr int K_BYTES = BN * K_RS;
+    static constexpr int V_RS = 2 * D + 64;   // bytes per V row in LDS
+    static constexpr int V_BYTES = BN * V_RS;
+    static constexpr int K_ITEMS = BN * (D / 16);  // 16-byte pieces per K tile
+    static constexpr int K_LOADS = (K_ITEMS + kFastThreads - 1) / kFastThreads;
+    static constexpr int V_LOADS = BN * (D / 8) / kFastThreads;
+    static constexpr int V_BASE = 2 * K_BYTES;
+    static constexpr int TOTAL = 2 * K_BYTES + 2 * V_BYTES;
+};
+
+template <typename VT>
+__device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0, const unsigned char* p1) {
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p1);
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(typename PV<VT>::vec, both);
+}
+
+template <int D, typename VT, bool CAUSAL>
+__global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
+    using F = FT<D>;
+    using PVT = PV<VT>;
+    using vec16 = typename PVT::vec;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+
+    // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
+    int wg = blockIdx.x;
+    if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
+    int iq = wg % nq2;
+    if (CAUSAL) iq = nq2 - 1 - iq;  // longest rows first
+    const int h = (wg / nq2) % a.Hq;
+    const int b = wg / (nq2 * a.Hq);
+    const int hk = h / a.groups;
+    const int m0 = iq * kFastRows;
+    const int my_m = m0 + 32 * wave + l32;
+    const bool row_ok = my_m < a.M;
+    const int shift = a.N - a.M;  // causal: key n is visible to row m iff n <= m + shift
+
+    int nsteps = a.nk;
+    if (CAUSAL) {
+        const int last_row = min(m0 + kFastRows, a.M) - 1;
+        nsteps = min(nsteps, (last_row + shift + BN) / BN);  // >= 1 because qo_len <= kv_len
+    }
+
+    // Q fragments: lane (row l32, half) holds channels half*D/2 + 16t .. +15 of k-step t
+    v4i qf[F::KSTEPS];
+    {
+        const int8_t* qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h + (int64_t)my_m * a.qs_n + half * (D / 2);
+#pragma unroll
+        for (int t = 0; t < F::KSTEPS; t++)
+            qf[t] = row_ok ? *reinterpret_cast<const v4i*>(qp + 16 * t) : v4i{0, 0, 0, 0};
+    }
+    const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + min(2 * iq + (wave >> 2), a.nq - 1)];
+    const float* ksp = a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk;
+    const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
+    const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
+
+    // staging: 16-byte pieces, consecutive lanes along a row
+    int k_goff[F::K_LOADS], k_lds[F::K_LOADS], v_goff[F::V_LOADS], v_lds[F::V_LOADS];
+    const bool k_worker = tid < F::K_ITEMS;
+#pragma unroll
+    for (int j = 0; j < F::K_LOADS; j++) {
+        const int id = (tid + kFastThreads * j) % F::K_ITEMS;
+        const int row = id / (D / 16), c = id % (D / 16);
+        k_goff[j] = row * (int)a.ks_n + 16 * c;
+        k_lds[j] = row * F::K_RS + 16 * c;
+    }
+#pragma unroll
+    for (int i = 0; i < F::V_LOADS; i++) {
+        const int id = tid + kFastThreads * i;
+        const int row = id / (D / 8), c = id % (D / 8);
+        v_goff[i] = row * (int)a.vs_n + 8 * c;
+        v_lds[i] = F::V_BASE + row * F::V_RS + 16 * c;
+    }
+    v4i kreg[F::K_LOADS];
+    v4i vreg[F::V_LOADS];  // native vectors: a struct type here ends up as a stack array in LDS
+    auto load_k = [&](int tile) {
+        const int8_t* kt = kg + (int64_t)tile * BN * a.ks_n;
+        if (k_worker) {
+#pragma unroll
+            for (int j = 0; j < F::K_LOADS; j++) kreg[j] = *reinterpret_cast<const v4i*>(kt + k_goff[j]);
+        }
+    };
+    auto load_v = [&](int tile) {
+        const VT* vt = vg + (int64_t)tile * BN * a.vs_n;
+#pragma unroll
+        for (int i = 0; i < F::V_LOADS; i++) vreg[i] = *reinterpret_cast<const v4i*>(vt + v_goff[i]);
+    };
+    auto store_k = [&](int buf) {
+        if (k_worker) {
+#pragma unroll
+            for (int j = 0; j < F::K_LOADS; j++) *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
+        }
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < F::V_LOADS; i++) *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
+    };
+
+    // fragment read offsets
+    const int kf_off = l32 * F::K_RS + 16 * half * (D / 32);
+    // ds_read_b64_tr_b16: in each group of 16 lanes, lane 4s+a supplies keys row s, channels 4a..4a+3,
+    // and lane i receives channel i of the four rows.  Groups: (channels 0-15 | 16-31) x (half 0 | 1).
+    const int vtr_off = F::V_BASE + (4 * half + ((lane >> 2) & 3)) * F::V_RS + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+    auto qk_tile = [&](const unsigned char* kbase, int kt) {
+        v16i acc;
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[i] = 0;
+#pragma unroll
+        for (int t = 0; t < F::KSTEPS; t++) {
+            const v4i kf = *reinterpret_cast<const v4i*>(kbase + kf_off + 32 * kt * F::K_RS + 16 * t);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[t], acc, 0, 0, 0);
+        }
+        return acc;
+    };
+
+    float m_i = -INFINITY;
+    float l_i = half ? 0.0f : 1.0f;  // the two halves of a row sum to the reference's initial l = 1
+    v16f o[F::DTILES];
+#pragma unroll
+    for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+
+    // ---- prologue: K0, V0, K1 in LDS; S of step 0 in registers
+    load_k(0);
+    load_v(0);
+    store_k(0);
+    store_v(0);
+    load_k(min(1, nsteps - 1));
+    store_k(1);
+    __syncthreads();
+    v16i s_cur[2];
+    s_cur[0] = qk_tile(smem, 0);
+    s_cur[1] = qk_tile(smem, 1);
+
+    for (int step = 0; step < nsteps; step++) {
+#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 5))
+#if defined(SAGE_ABL) && SAGE_ABL == 6
+        load_k(0);
+        load_v(0);
+#else
+        load_k(min(step + 2, nsteps - 1));
+        load_v(min(step + 1, nsteps - 1));
+#endif
+#endif
+        __builtin_amdgcn_sched_barrier(0);  // the fetches go out first ...
+        const int n0 = step * BN;
+        const unsigned char* kb_next = smem + ((step + 1) & 1) * F::K_BYTES;
+        const unsigned char* vb_cur = smem + (step & 1) * F::V_BYTES + vtr_off;
+
+        // ---- row maximum of step `step` (runs while P.V of the previous step drains)
+        float f[2][16];
+        float rmax = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) f[kt][i] = (float)s_cur[kt][i];
+        bool diag = false;
+        if (CAUSAL) diag = n0 + BN - 1 > m0 + 32 * wave + shift;  // some element of this wave's tile is hidden
+        if (CAUSAL && diag) {
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
+                    if (n > my_m + shift) f[kt][i] = -INFINITY;
+                }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) rmax = fmaxf(rmax, f[kt][i]);
+        const float sc = qs * ksp[step];
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 32)) * sc;
+        const float m_new = fmaxf(m_i, rmax);
+        if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+            l_i *= alpha;
+            m_i = m_new;
+#pragma unroll
+            for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+        const float neg_m = -m_i;
+
+        // ---- Q.K^T of the next step on the matrix core, exponentials of this step on the VALU
+        v16i s_next[2];
+        s_next[0] = qk_tile(kb_next, 0);
+        s_next[1] = qk_tile(kb_next, 1);
+
+        vec16 pf[4];
+        float lsum = 0.0f;
+#pragma unroll
+        for (int tp = 0; tp < 4; tp++) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+#if defined(SAGE_ABL) && SAGE_ABL == 2
+                float p = __builtin_fmaf(f[tp >> 1][8 * (tp & 1) + c], sc, neg_m);
+#else
+                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(f[tp >> 1][8 * (tp & 1) + c], sc, neg_m));
+#endif
+                if (CAUSAL && diag) {
+                    const int n = n0 + 16 * tp + 8 * (c >> 2) + 4 * half + (c & 3);
+                    p = (n > my_m + shift) ? 0.0f : p;
+                }
+                pf[tp][c] = (VT)p;
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) lsum = PVT::dot2_ones(pf[tp], c, lsum);
+        }
+        l_i += lsum;
+
+        // ---- O^T += V^T . P^T
+#pragma unroll
+        for (int tp = 0; tp < 4; tp++)
+#pragma unroll
+            for (int dt = 0; dt < F::DTILES; dt++) {
+                const unsigned char* p0 = vb_cur + (16 * tp) * F::V_RS + 64 * dt;
+#if defined(SAGE_ABL) && SAGE_ABL == 1
+                const vec16 vf = *reinterpret_cast<const vec16*>(p0);
+#else
+                const vec16 vf = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+#endif
+                o[dt] = PVT::mfma(vf, pf[tp], o[dt]);
+            }
+
+        s_cur[0] = s_next[0];
+        s_cur[1] = s_next[1];
+        __builtin_amdgcn_sched_barrier(0);  // ... and are only waited for after the math of this step
+#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 5))
+        store_k(step & 1);
+        store_v((step + 1) & 1);
+#endif
+#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 4))
+        __syncthreads();
+#endif
+    }
+
+    // ---- epilogue: O = O^T / l, lse = log2(l) + m
+    const float l_o = __shfl_xor(l_i, 32);
+    const float l_tot = half ? (l_o + l_i) : (l_i + l_o);
+    const float inv = 1.0f / l_tot;
+    if (row_ok) {
+        const int64_t obase = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)my_m * a.os_n;
+#pragma unroll
+        for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d = 32 * dt + 8 * g + 4 * half;
+                float r[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] = o[dt][4 * g + i] * inv;
+                if (a.out_dt == SAGE_BF16) {
+                    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+                    b4 w = {(__bf16)r[0], (__bf16)r[1], (__bf16)r[2], (__bf16)r[3]};
+                    *reinterpret_cast<b4*>(static_cast<__bf16*>(a.out) + obase + d) = w;
+                } else if (a.out_dt == SAGE_F16) {
+                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                    h4 w = {(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
+                    *reinterpret_cast<h4*>(static_cast<_Float16*>(a.out) + obase + d) = w;
+                } else {
+                    *reinterpret_cast<v4f*>(static_cast<float*>(a.out) + obase + d) = v4f{r[0], r[1], r[2], r[3]};
+                }
+            }
+        if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
+    }
+}
+
+template <int D, typename VT>
+int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
+    AttnArgs b = a;
+    const int nq2 = (a.M + kFastRows - 1) / kFastRows;
+    b.total_wg = (int)((int64_t)a.total_wg / a.nq * nq2);
+    dim3 grid((unsigned)b.total_wg), block(kFastThreads);
+    if (causal) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true>), grid, block, 0, stream, b, nq2);
+    else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false>), grid, block, 0, stream, b, nq2);
+    return check_launch("sage_attn_fwd_fast_kernel");
+}
+
+}  // namespace
+
+int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream) {
+    if (head_dim == 128)
+        return v_dtype == SAGE_BF16 ? launch_causal<128, __bf16>(a, causal, stream)
+                                    : launch_causal<128, _Float16>(a, causal, stream);
+    return v_dtype == SAGE_BF16 ? launch_causal<64, __bf16>(a, causal, stream)
+                                : launch_causal<64, _Float16>(a, causal, stream);
+}
+
+}  // namespace attn
+}  // namespace sage
