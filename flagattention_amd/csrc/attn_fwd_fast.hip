@@ -17,6 +17,8 @@
 //   into registers at the top of iteration j and stored to LDS at its end (one barrier per step).
 // * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
 //   rare steps where a row maximum jumps.
+#include <utility>
+
 #include "attn_common.h"
 
 namespace sage {
@@ -26,6 +28,14 @@ namespace {
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+// compile-time loops: f(IC<0>{}), f(IC<1>{}), ...
+template <int I> struct IC { static constexpr int value = I; };
+template <typename Fn, int... Is>
+__device__ __forceinline__ void sfor_impl(Fn&& f, std::integer_sequence<int, Is...>) { (f(IC<Is>{}), ...); }
+template <int N, typename Fn>
+__device__ __forceinline__ void sfor(Fn&& f) { sfor_impl(f, std::make_integer_sequence<int, N>{}); }
 
 constexpr int kFastThreads = 512;  // 8 waves
 constexpr int kFastRows = 256;     // query rows per workgroup
@@ -119,7 +129,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     v4i vreg[F::V_LOADS];  // native vectors: a struct type here ends up as a stack array in LDS
     auto load_k = [&](int tile) {
         const int8_t* kt = kg + (int64_t)tile * BN * a.ks_n;
-        if (k_worker) {
+        if (F::K_ITEMS >= kFastThreads || k_worker) {
 #pragma unroll
             for (int j = 0; j < F::K_LOADS; j++) kreg[j] = *reinterpret_cast<const v4i*>(kt + k_goff[j]);
         }
@@ -130,7 +140,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         for (int i = 0; i < F::V_LOADS; i++) vreg[i] = *reinterpret_cast<const v4i*>(vt + v_goff[i]);
     };
     auto store_k = [&](int buf) {
-        if (k_worker) {
+        if (F::K_ITEMS >= kFastThreads || k_worker) {
 #pragma unroll
             for (int j = 0; j < F::K_LOADS; j++) *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
         }
@@ -166,7 +176,48 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
 #pragma unroll
         for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
 
-    // ---- prologue: K0, V0, K1 in LDS; S of step 0 in registers
+    // ---- the step pipeline -----------------------------------------------------------------
+    // One iteration issues QK_SLOTS + PV_SLOTS matrix instructions.  Each "slot" is one MFMA plus
+    // the VALU work that runs in its shadow, fenced so that the order written here is the order
+    // issued:
+    //   E(u), u = 0..15: two scores of the CURRENT step -> exp2 -> 16-bit pair of P -> row sum
+    //   H(u), u = 0..7 : four scores of the NEXT step (whose Q.K^T finished earlier in this very
+    //                    iteration) -> fp32 -> running raw maximum
+    // LDS fragment reads are issued a few slots ahead of the MFMA that consumes them.
+    constexpr int QK_SLOTS = 2 * F::KSTEPS;
+    constexpr int PV_SLOTS = 4 * F::DTILES;
+    constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
+    constexpr int UPS = 24 / NSLOTS;  // units per slot
+    constexpr int KDIST = 4;          // K fragments in flight
+    constexpr int VDIST = 3;          // V fragments in flight
+    static_assert(UPS * NSLOTS == 24 && KDIST <= QK_SLOTS && VDIST < QK_SLOTS, "slot plan");
+
+    float f[2][16];   // raw scores of the current step as fp32
+    float raw_max;    // their maximum over this lane's 32 keys (before the block scale)
+    float sc;         // q_scale * k_scale of the current step
+    v16i s_next[2];
+    float fn[2][16];
+    float raw_max_n;
+
+    auto head_unit = [&](auto uc, int n0_next, bool masked) {
+        constexpr int u = decltype(uc)::value;
+        constexpr int kt = u >> 2, i0 = 4 * (u & 3);
+#pragma unroll
+        for (int i = i0; i < i0 + 4; i++) {
+            float x = (float)s_next[kt][i];
+            if (CAUSAL && masked) {
+                const int n = n0_next + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
+                x = (n > my_m + shift) ? -INFINITY : x;
+            }
+            fn[kt][i] = x;
+        }
+        raw_max_n = fmaxf(fmaxf(raw_max_n, fn[kt][i0]), fn[kt][i0 + 1]);
+        raw_max_n = fmaxf(fmaxf(raw_max_n, fn[kt][i0 + 2]), fn[kt][i0 + 3]);
+        // pin the results to this slot (otherwise they are sunk below the matrix instructions)
+        asm volatile("" ::"v"(raw_max_n), "v"(fn[kt][i0]), "v"(fn[kt][i0 + 1]), "v"(fn[kt][i0 + 2]), "v"(fn[kt][i0 + 3]));
+    };
+
+    // ---- prologue: K0, V0, K1 in LDS; scores of step 0 in registers
     load_k(0);
     load_v(0);
     store_k(0);
@@ -174,112 +225,120 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     load_k(min(1, nsteps - 1));
     store_k(1);
     __syncthreads();
-    v16i s_cur[2];
-    s_cur[0] = qk_tile(smem, 0);
-    s_cur[1] = qk_tile(smem, 1);
+    s_next[0] = qk_tile(smem, 0);
+    s_next[1] = qk_tile(smem, 1);
+    raw_max_n = -INFINITY;
+    {
+        const bool masked0 = CAUSAL && (BN - 1 > m0 + 32 * wave + shift);
+        sfor<8>([&](auto uc) { head_unit(uc, 0, masked0); });
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) f[kt][i] = fn[kt][i];
+    raw_max = raw_max_n;
+    sc = qs * ksp[0];
+    if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
 
     for (int step = 0; step < nsteps; step++) {
-#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 5))
-#if defined(SAGE_ABL) && SAGE_ABL == 6
-        load_k(0);
-        load_v(0);
-#else
         load_k(min(step + 2, nsteps - 1));
         load_v(min(step + 1, nsteps - 1));
-#endif
-#endif
-        __builtin_amdgcn_sched_barrier(0);  // the fetches go out first ...
-        const int n0 = step * BN;
-        const unsigned char* kb_next = smem + ((step + 1) & 1) * F::K_BYTES;
+        const unsigned char* kb_next = smem + ((step + 1) & 1) * F::K_BYTES + kf_off;
         const unsigned char* vb_cur = smem + (step & 1) * F::V_BYTES + vtr_off;
+        const int n0_next = (step + 1) * BN;
+        float sc_n = qs * ksp[min(step + 1, nsteps - 1)];
+        if (CAUSAL) sc_n = fmaxf(sc_n, 1.17549435e-38f);
+        const bool masked_n = CAUSAL && (n0_next + BN - 1 > m0 + 32 * wave + shift);
 
-        // ---- row maximum of step `step` (runs while P.V of the previous step drains)
-        float f[2][16];
-        float rmax = -INFINITY;
+        v4i kfr[QK_SLOTS];
+        vec16 vfr[PV_SLOTS];
+        auto read_k = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            kfr[i] = *reinterpret_cast<const v4i*>(kb_next + 32 * (i / F::KSTEPS) * F::K_RS + 16 * (i % F::KSTEPS));
+        };
+        auto read_v = [&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const unsigned char* p0 = vb_cur + 16 * (j / F::DTILES) * F::V_RS + 64 * (j % F::DTILES);
+            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+        };
+        sfor<KDIST>(read_k);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- finish the row maximum of this step; advance the running maximum only on a jump
+        {
+            const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, raw_max),
+                                                            __builtin_bit_cast(unsigned, raw_max), false, false);
+            const float rmax = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) * sc;
+            const float m_new = fmaxf(m_i, rmax);
+            if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+                l_i *= alpha;
+                m_i = m_new;
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+                for (int dt = 0; dt < F::DTILES; dt++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) f[kt][i] = (float)s_cur[kt][i];
-        bool diag = false;
-        if (CAUSAL) diag = n0 + BN - 1 > m0 + 32 * wave + shift;  // some element of this wave's tile is hidden
-        if (CAUSAL && diag) {
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
-                    if (n > my_m + shift) f[kt][i] = -INFINITY;
-                }
-        }
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) rmax = fmaxf(rmax, f[kt][i]);
-        const float sc = qs * ksp[step];
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 32)) * sc;
-        const float m_new = fmaxf(m_i, rmax);
-        if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
-            const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-            l_i *= alpha;
-            m_i = m_new;
-#pragma unroll
-            for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+            }
         }
         const float neg_m = -m_i;
-
-        // ---- Q.K^T of the next step on the matrix core, exponentials of this step on the VALU
-        v16i s_next[2];
-        s_next[0] = qk_tile(kb_next, 0);
-        s_next[1] = qk_tile(kb_next, 1);
-
         vec16 pf[4];
         float lsum = 0.0f;
+        raw_max_n = -INFINITY;
+        __builtin_amdgcn_sched_barrier(0);
+
+        auto exp_unit = [&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(f[kt][i0], sc, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(f[kt][i0 + 1], sc, neg_m));
+            pf[tp][2 * w] = (VT)p0;
+            pf[tp][2 * w + 1] = (VT)p1;
+            lsum = PVT::dot2_ones(pf[tp], w, lsum);
+            asm volatile("" ::"v"(lsum));  // pin to this slot
+        };
+        auto slots = [&](auto maskc) {
+            constexpr bool MASKED = decltype(maskc)::value != 0;
+            sfor<NSLOTS>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i < QK_SLOTS) {
+                    constexpr int kt = i / F::KSTEPS, t = i % F::KSTEPS;
+                    if constexpr (t == 0) {
+                        v16i z;
 #pragma unroll
-        for (int tp = 0; tp < 4; tp++) {
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-#if defined(SAGE_ABL) && SAGE_ABL == 2
-                float p = __builtin_fmaf(f[tp >> 1][8 * (tp & 1) + c], sc, neg_m);
-#else
-                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(f[tp >> 1][8 * (tp & 1) + c], sc, neg_m));
-#endif
-                if (CAUSAL && diag) {
-                    const int n = n0 + 16 * tp + 8 * (c >> 2) + 4 * half + (c & 3);
-                    p = (n > my_m + shift) ? 0.0f : p;
+                        for (int e = 0; e < 16; e++) z[e] = 0;
+                        s_next[kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], z, 0, 0, 0);
+                    } else {
+                        s_next[kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], s_next[kt], 0, 0, 0);
+                    }
+                    if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
+                    if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
+                } else {
+                    constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
+                    o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
+                    if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
                 }
-                pf[tp][c] = (VT)p;
-            }
-#pragma unroll
-            for (int c = 0; c < 4; c++) lsum = PVT::dot2_ones(pf[tp], c, lsum);
-        }
+                sfor<UPS>([&](auto rc) {
+                    constexpr int u = i * UPS + decltype(rc)::value;
+                    if constexpr (u < 16) exp_unit(IC<u>{});
+                    else head_unit(IC<u - 16>{}, n0_next, MASKED);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        if (CAUSAL && masked_n) slots(IC<1>{});
+        else slots(IC<0>{});
+
         l_i += lsum;
-
-        // ---- O^T += V^T . P^T
 #pragma unroll
-        for (int tp = 0; tp < 4; tp++)
+        for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-            for (int dt = 0; dt < F::DTILES; dt++) {
-                const unsigned char* p0 = vb_cur + (16 * tp) * F::V_RS + 64 * dt;
-#if defined(SAGE_ABL) && SAGE_ABL == 1
-                const vec16 vf = *reinterpret_cast<const vec16*>(p0);
-#else
-                const vec16 vf = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
-#endif
-                o[dt] = PVT::mfma(vf, pf[tp], o[dt]);
-            }
-
-        s_cur[0] = s_next[0];
-        s_cur[1] = s_next[1];
-        __builtin_amdgcn_sched_barrier(0);  // ... and are only waited for after the math of this step
-#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 5))
+            for (int i = 0; i < 16; i++) f[kt][i] = fn[kt][i];
+        raw_max = raw_max_n;
+        sc = sc_n;
+        __builtin_amdgcn_sched_barrier(0);  // the fetched tiles are only waited for after the math of this step
         store_k(step & 1);
         store_v((step + 1) & 1);
-#endif
-#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 4))
         __syncthreads();
-#endif
     }
 
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
