@@ -37,6 +37,11 @@ __device__ __forceinline__ void sfor_impl(Fn&& f, std::integer_sequence<int, Is.
 template <int N, typename Fn>
 __device__ __forceinline__ void sfor(Fn&& f) { sfor_impl(f, std::make_integer_sequence<int, N>{}); }
 
+constexpr int kBiasBits = 0x4B400000;  // 12582912.0f = 1.5 * 2^23
+constexpr float kBias = 12582912.0f;
+// exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
+// product the bias is subtracted explicitly instead.
+constexpr float kBiasFoldLimit = 8192.0f;
 constexpr int kFastThreads = 512;  // 8 waves
 constexpr int kFastRows = 256;     // query rows per workgroup
 
@@ -156,10 +161,13 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     // and lane i receives channel i of the four rows.  Groups: (channels 0-15 | 16-31) x (half 0 | 1).
     const int vtr_off = F::V_BASE + (4 * half + ((lane >> 2) & 3)) * F::V_RS + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
-    auto qk_tile = [&](const unsigned char* kbase, int kt) {
-        v16i acc;
+    // The int32 accumulators start from the bit pattern of the float 1.5 * 2^23: since |dot| < 2^22,
+    // accumulator bits reinterpreted as fp32 ARE kBias + dot, so no int -> float conversion is needed.
+    v16i bias16;
 #pragma unroll
-        for (int i = 0; i < 16; i++) acc[i] = 0;
+    for (int i = 0; i < 16; i++) bias16[i] = kBiasBits;
+    auto qk_tile = [&](const unsigned char* kbase, int kt) {
+        v16i acc = bias16;
 #pragma unroll
         for (int t = 0; t < F::KSTEPS; t++) {
             const v4i kf = *reinterpret_cast<const v4i*>(kbase + kf_off + 32 * kt * F::K_RS + 16 * t);
@@ -188,33 +196,42 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
     constexpr int UPS = 24 / NSLOTS;  // units per slot
-    constexpr int KDIST = 4;          // K fragments in flight
-    constexpr int VDIST = 3;          // V fragments in flight
+#ifndef SAGE_KDIST
+#define SAGE_KDIST 4
+#endif
+#ifndef SAGE_VDIST
+#define SAGE_VDIST 3
+#endif
+    constexpr int KDIST = SAGE_KDIST < QK_SLOTS ? SAGE_KDIST : QK_SLOTS;  // K fragments in flight
+    constexpr int VDIST = SAGE_VDIST < QK_SLOTS ? SAGE_VDIST : QK_SLOTS - 1;  // V fragments in flight
     static_assert(UPS * NSLOTS == 24 && KDIST <= QK_SLOTS && VDIST < QK_SLOTS, "slot plan");
 
-    float f[2][16];   // raw scores of the current step as fp32
-    float raw_max;    // their maximum over this lane's 32 keys (before the block scale)
+    // Scores live in two register sets that swap roles every step (the loop body is instantiated
+    // for both parities), so the accumulators Q.K^T writes in one iteration are read in place by
+    // the exponentials of the next one.
+    v16i sbuf[2][2];  // [parity][32-key tile]: int32 accumulators whose bits are the float kBias + dot
+    float raw_max;    // maximum of the current step's 32 biased scores of this lane
     float sc;         // q_scale * k_scale of the current step
-    v16i s_next[2];
-    float fn[2][16];
-    float raw_max_n;
 
-    auto head_unit = [&](auto uc, int n0_next, bool masked) {
-        constexpr int u = decltype(uc)::value;
+    auto as_f = [](int bits) { return __builtin_bit_cast(float, bits); };
+    auto head_unit = [&](auto pc, auto uc, int n0_next, bool masked, float& acc) {
+        constexpr int P = decltype(pc)::value, u = decltype(uc)::value;
         constexpr int kt = u >> 2, i0 = 4 * (u & 3);
+        float x[4];
 #pragma unroll
-        for (int i = i0; i < i0 + 4; i++) {
-            float x = (float)s_next[kt][i];
+        for (int e = 0; e < 4; e++) {
+            const int bits = sbuf[P][kt][i0 + e];  // (scalar copy: bit_cast of a vector element lvalue reads element 0)
+            x[e] = as_f(bits);
             if (CAUSAL && masked) {
+                const int i = i0 + e;
                 const int n = n0_next + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
-                x = (n > my_m + shift) ? -INFINITY : x;
+                x[e] = (n > my_m + shift) ? -INFINITY : x[e];
+                sbuf[P][kt][i] = __builtin_bit_cast(int, x[e]);
             }
-            fn[kt][i] = x;
         }
-        raw_max_n = fmaxf(fmaxf(raw_max_n, fn[kt][i0]), fn[kt][i0 + 1]);
-        raw_max_n = fmaxf(fmaxf(raw_max_n, fn[kt][i0 + 2]), fn[kt][i0 + 3]);
-        // pin the results to this slot (otherwise they are sunk below the matrix instructions)
-        asm volatile("" ::"v"(raw_max_n), "v"(fn[kt][i0]), "v"(fn[kt][i0 + 1]), "v"(fn[kt][i0 + 2]), "v"(fn[kt][i0 + 3]));
+        acc = fmaxf(fmaxf(acc, x[0]), x[1]);
+        acc = fmaxf(fmaxf(acc, x[2]), x[3]);
+        asm volatile("" ::"v"(acc));  // pin to this slot (otherwise sunk below the matrix instructions)
     };
 
     // ---- prologue: K0, V0, K1 in LDS; scores of step 0 in registers
@@ -225,26 +242,30 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     load_k(min(1, nsteps - 1));
     store_k(1);
     __syncthreads();
-    s_next[0] = qk_tile(smem, 0);
-    s_next[1] = qk_tile(smem, 1);
-    raw_max_n = -INFINITY;
+    sbuf[0][0] = qk_tile(smem, 0);
+    sbuf[0][1] = qk_tile(smem, 1);
+    raw_max = -INFINITY;
     {
         const bool masked0 = CAUSAL && (BN - 1 > m0 + 32 * wave + shift);
-        sfor<8>([&](auto uc) { head_unit(uc, 0, masked0); });
+        sfor<8>([&](auto uc) { head_unit(IC<0>{}, uc, 0, masked0, raw_max); });
     }
-#pragma unroll
-    for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) f[kt][i] = fn[kt][i];
-    raw_max = raw_max_n;
     sc = qs * ksp[0];
     if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
 
-    for (int step = 0; step < nsteps; step++) {
+#ifdef SAGE_PROF
+    long long prof[4] = {0, 0, 0, 0};
+#define PROF_T(v) const long long v = __builtin_readcyclecounter(); asm volatile("" ::: "memory")
+#else
+#define PROF_T(v)
+#endif
+
+    auto body = [&](auto pc, int step) {
+        constexpr int P = decltype(pc)::value;  // == step & 1
+        PROF_T(t_top);
         load_k(min(step + 2, nsteps - 1));
         load_v(min(step + 1, nsteps - 1));
-        const unsigned char* kb_next = smem + ((step + 1) & 1) * F::K_BYTES + kf_off;
-        const unsigned char* vb_cur = smem + (step & 1) * F::V_BYTES + vtr_off;
+        const unsigned char* kb_next = smem + (1 - P) * F::K_BYTES + kf_off;
+        const unsigned char* vb_cur = smem + P * F::V_BYTES + vtr_off;
         const int n0_next = (step + 1) * BN;
         float sc_n = qs * ksp[min(step + 1, nsteps - 1)];
         if (CAUSAL) sc_n = fmaxf(sc_n, 1.17549435e-38f);
@@ -268,7 +289,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         {
             const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, raw_max),
                                                             __builtin_bit_cast(unsigned, raw_max), false, false);
-            const float rmax = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) * sc;
+            const float rmax = (fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) - kBias) * sc;
             const float m_new = fmaxf(m_i, rmax);
             if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
                 const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
@@ -280,17 +301,31 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                     for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
             }
         }
-        const float neg_m = -m_i;
+        float neg_m;  // exponent of a score with biased bits x: fma(x, sc, neg_m)
+        if (kBias * sc < kBiasFoldLimit) {
+            neg_m = __builtin_fmaf(-kBias, sc, -m_i);
+        } else {  // large block scales: remove the bias first (exact), keep full precision
+#pragma unroll
+            for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int bits = sbuf[P][kt][i];
+                    sbuf[P][kt][i] = __builtin_bit_cast(int, as_f(bits) - kBias);
+                }
+            neg_m = -m_i;
+        }
         vec16 pf[4];
         float lsum = 0.0f;
-        raw_max_n = -INFINITY;
+        float raw_max_n = -INFINITY;
         __builtin_amdgcn_sched_barrier(0);
+        PROF_T(t_head);
 
         auto exp_unit = [&](auto uc) {
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(f[kt][i0], sc, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(f[kt][i0 + 1], sc, neg_m));
+            const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc, neg_m));
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
             lsum = PVT::dot2_ones(pf[tp], w, lsum);
@@ -303,12 +338,9 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                 if constexpr (i < QK_SLOTS) {
                     constexpr int kt = i / F::KSTEPS, t = i % F::KSTEPS;
                     if constexpr (t == 0) {
-                        v16i z;
-#pragma unroll
-                        for (int e = 0; e < 16; e++) z[e] = 0;
-                        s_next[kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], z, 0, 0, 0);
+                        sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], bias16, 0, 0, 0);
                     } else {
-                        s_next[kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], s_next[kt], 0, 0, 0);
+                        sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
                     }
                     if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
                     if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
@@ -320,7 +352,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                 sfor<UPS>([&](auto rc) {
                     constexpr int u = i * UPS + decltype(rc)::value;
                     if constexpr (u < 16) exp_unit(IC<u>{});
-                    else head_unit(IC<u - 16>{}, n0_next, MASKED);
+                    else head_unit(IC<1 - P>{}, IC<u - 16>{}, n0_next, MASKED, raw_max_n);
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -329,17 +361,34 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         else slots(IC<0>{});
 
         l_i += lsum;
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) f[kt][i] = fn[kt][i];
         raw_max = raw_max_n;
         sc = sc_n;
         __builtin_amdgcn_sched_barrier(0);  // the fetched tiles are only waited for after the math of this step
-        store_k(step & 1);
-        store_v((step + 1) & 1);
+        PROF_T(t_slots);
+        store_k(P);
+        store_v(1 - P);
+        PROF_T(t_store);
         __syncthreads();
+#ifdef SAGE_PROF
+        {
+            PROF_T(t_end);
+            prof[0] += t_head - t_top; prof[1] += t_slots - t_head; prof[2] += t_store - t_slots; prof[3] += t_end - t_store;
+        }
+#endif
+    };
+
+    for (int step = 0; step < nsteps; step += 2) {
+        body(IC<0>{}, step);
+        if (step + 1 >= nsteps) break;
+        body(IC<1>{}, step + 1);
     }
+#ifdef SAGE_PROF
+    if (a.lse && lane == 0) {
+        float* dst = a.lse + ((int64_t)blockIdx.x * 8 + wave) * 4;
+        for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
+    }
+    return;
+#endif
 
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
     const float l_o = __shfl_xor(l_i, 32);
