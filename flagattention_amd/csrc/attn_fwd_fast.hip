@@ -13,8 +13,9 @@
 //   the A operand of the P.V MFMA, with no shuffling instructions.
 // * The loop is skewed by one step: while the exponentials of step j run on the VALU, the matrix
 //   core works on Q.K^T of step j+1 and then on P.V of step j, whose tail overlaps the row-max
-//   pass of the next iteration.  K of step j+2 and V of step j+1 are fetched from global memory
-//   into registers at the top of iteration j and stored to LDS at its end (one barrier per step).
+//   pass of the next iteration.  K of step j+3 and V of step j+2 are fetched from global memory
+//   into registers at the top of iteration j and stored to LDS at the top of iteration j+1 (one
+//   barrier per step, nothing to drain in front of it).
 // * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
 //   rare steps where a row maximum jumps.
 #include <utility>
@@ -242,6 +243,8 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     load_k(min(1, nsteps - 1));
     store_k(1);
     __syncthreads();
+    load_k(min(2, nsteps - 1));  // stored to LDS at the top of the first iteration
+    load_v(min(1, nsteps - 1));
     sbuf[0][0] = qk_tile(smem, 0);
     sbuf[0][1] = qk_tile(smem, 1);
     raw_max = -INFINITY;
@@ -262,8 +265,21 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     auto body = [&](auto pc, int step) {
         constexpr int P = decltype(pc)::value;  // == step & 1
         PROF_T(t_top);
-        load_k(min(step + 2, nsteps - 1));
-        load_v(min(step + 1, nsteps - 1));
+        // K of step+2 and V of step+1 were fetched into registers during the previous iteration:
+        // hand them to LDS now (their buffers were released by the barrier that ended it) and
+        // start fetching the tiles after them, so neither the fetch nor the LDS write is waited
+        // for at the end of a step.
+#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 12 || SAGE_ABL == 5))
+        store_k(P);
+        store_v(1 - P);
+#if defined(SAGE_ABL) && SAGE_ABL == 6
+        load_k(0);
+        load_v(0);
+#else
+        load_k(min(step + 3, nsteps - 1));
+        load_v(min(step + 2, nsteps - 1));
+#endif
+#endif
         const unsigned char* kb_next = smem + (1 - P) * F::K_BYTES + kf_off;
         const unsigned char* vb_cur = smem + P * F::V_BYTES + vtr_off;
         const int n0_next = (step + 1) * BN;
@@ -275,12 +291,32 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         vec16 vfr[PV_SLOTS];
         auto read_k = [&](auto ic) {
             constexpr int i = decltype(ic)::value;
+#if defined(SAGE_ABL) && (SAGE_ABL == 10 || SAGE_ABL == 12)
+            kfr[i] = qf[(i + 1) % F::KSTEPS];
+            (void)kb_next;
+#else
             kfr[i] = *reinterpret_cast<const v4i*>(kb_next + 32 * (i / F::KSTEPS) * F::K_RS + 16 * (i % F::KSTEPS));
+#endif
         };
         auto read_v = [&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const unsigned char* p0 = vb_cur + 16 * (j / F::DTILES) * F::V_RS + 64 * (j % F::DTILES);
+#if defined(SAGE_ABL) && (SAGE_ABL == 10 || SAGE_ABL == 12)
+            vfr[j] = __builtin_bit_cast(vec16, qf[j % F::KSTEPS]);
+            (void)p0;
+#elif defined(SAGE_ABL) && SAGE_ABL == 13
+            {
+                typedef int v2i __attribute__((ext_vector_type(2)));
+                const v2i lo = *reinterpret_cast<const v2i*>(p0), hi = *reinterpret_cast<const v2i*>(p0 + 8 * F::V_RS);
+                const v4i both = {lo[0], lo[1], hi[0], hi[1]};
+                vfr[j] = __builtin_bit_cast(vec16, both);
+            }
+#elif defined(SAGE_ABL) && SAGE_ABL == 14
+            vfr[j] = *reinterpret_cast<const vec16*>(smem + F::V_BASE + P * F::V_BYTES + (lane & 31) * 272 + (lane >> 5) * 16 + (j % 8) * 32 + (j / 8) * 8704);
+            (void)p0;
+#else
             vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+#endif
         };
         sfor<KDIST>(read_k);
         __builtin_amdgcn_sched_barrier(0);
@@ -335,6 +371,16 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
             constexpr bool MASKED = decltype(maskc)::value != 0;
             sfor<NSLOTS>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
+#ifdef SAGE_PRIO
+                // The two waves that share a SIMD trade issue priority halfway through the step so
+                // that they reach the barrier together.
+                if constexpr (i == 0) {
+                    if (wave < 4) __builtin_amdgcn_s_setprio(SAGE_PRIO); else __builtin_amdgcn_s_setprio(0);
+                }
+                if constexpr (i == NSLOTS / 2) {
+                    if (wave < 4) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(SAGE_PRIO);
+                }
+#endif
                 if constexpr (i < QK_SLOTS) {
                     constexpr int kt = i / F::KSTEPS, t = i % F::KSTEPS;
                     if constexpr (t == 0) {
@@ -365,10 +411,10 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         sc = sc_n;
         __builtin_amdgcn_sched_barrier(0);  // the fetched tiles are only waited for after the math of this step
         PROF_T(t_slots);
-        store_k(P);
-        store_v(1 - P);
         PROF_T(t_store);
+#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 12))
         __syncthreads();
+#endif
 #ifdef SAGE_PROF
         {
             PROF_T(t_end);
@@ -382,13 +428,6 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         if (step + 1 >= nsteps) break;
         body(IC<1>{}, step + 1);
     }
-#ifdef SAGE_PROF
-    if (a.lse && lane == 0) {
-        float* dst = a.lse + ((int64_t)blockIdx.x * 8 + wave) * 4;
-        for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
-    }
-    return;
-#endif
 
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
     const float l_o = __shfl_xor(l_i, 32);
@@ -416,8 +455,16 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                     *reinterpret_cast<v4f*>(static_cast<float*>(a.out) + obase + d) = v4f{r[0], r[1], r[2], r[3]};
                 }
             }
+#ifndef SAGE_PROF
         if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
+#endif
     }
+#ifdef SAGE_PROF
+    if (a.lse && lane == 0) {  // debug build: per-wave cycle totals of the loop phases replace the lse output
+        float* dst = a.lse + ((int64_t)blockIdx.x * 8 + wave) * 4;
+        for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
+    }
+#endif
 }
 
 template <int D, typename VT>
