@@ -151,6 +151,19 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
             for (int j = 0; j < F::K_LOADS; j++) *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
         }
     };
+    // piecewise variants used inside the step pipeline (one 16-byte piece per call)
+    auto restage_k = [&](auto jc, int buf, int tile) {
+        constexpr int j = decltype(jc)::value;
+        if (F::K_ITEMS >= kFastThreads || k_worker) {
+            *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
+            kreg[j] = *reinterpret_cast<const v4i*>(kg + (int64_t)tile * BN * a.ks_n + k_goff[j]);
+        }
+    };
+    auto restage_v = [&](auto ic, int buf, int tile) {
+        constexpr int i = decltype(ic)::value;
+        *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
+        vreg[i] = *reinterpret_cast<const v4i*>(vg + (int64_t)tile * BN * a.vs_n + v_goff[i]);
+    };
     auto store_v = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < F::V_LOADS; i++) *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
@@ -265,21 +278,6 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     auto body = [&](auto pc, int step) {
         constexpr int P = decltype(pc)::value;  // == step & 1
         PROF_T(t_top);
-        // K of step+2 and V of step+1 were fetched into registers during the previous iteration:
-        // hand them to LDS now (their buffers were released by the barrier that ended it) and
-        // start fetching the tiles after them, so neither the fetch nor the LDS write is waited
-        // for at the end of a step.
-#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 12 || SAGE_ABL == 5))
-        store_k(P);
-        store_v(1 - P);
-#if defined(SAGE_ABL) && SAGE_ABL == 6
-        load_k(0);
-        load_v(0);
-#else
-        load_k(min(step + 3, nsteps - 1));
-        load_v(min(step + 2, nsteps - 1));
-#endif
-#endif
         const unsigned char* kb_next = smem + (1 - P) * F::K_BYTES + kf_off;
         const unsigned char* vb_cur = smem + P * F::V_BYTES + vtr_off;
         const int n0_next = (step + 1) * BN;
@@ -394,6 +392,12 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                     constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                     o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
                     if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
+                    // K of step+2 and V of step+1 were fetched into registers during the previous
+                    // iteration: hand one piece per slot to LDS (those buffers were released by the
+                    // barrier that ended it) and refill the register with the tile after it.  Neither
+                    // the fetch nor the LDS write is waited for at the end of a step.
+                    if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, min(step + 3, nsteps - 1));
+                    else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, min(step + 2, nsteps - 1));
                 }
                 sfor<UPS>([&](auto rc) {
                     constexpr int u = i * UPS + decltype(rc)::value;
