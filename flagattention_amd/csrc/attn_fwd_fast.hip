@@ -11,11 +11,17 @@
 // * V is staged in LDS as it lies in memory ([key][channel], rows padded by 64 bytes) and read
 //   with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel: exactly
 //   the A operand of the P.V MFMA, with no shuffling instructions.
-// * The loop is skewed by one step: while the exponentials of step j run on the VALU, the matrix
-//   core works on Q.K^T of step j+1 and then on P.V of step j, whose tail overlaps the row-max
-//   pass of the next iteration.  K of step j+3 and V of step j+2 are fetched from global memory
-//   into registers at the top of iteration j and stored to LDS at the top of iteration j+1 (one
-//   barrier per step, nothing to drain in front of it).
+// * Every wave alternates between a VALU phase (exponentials of step j) and an MFMA phase (Q.K^T of
+//   step j+1 and P.V of step j back to back, with the row sums of P and the raw row maximum of
+//   step j+1 riding in the shadow of the matrix instructions).  The two waves that share a SIMD
+//   run half a step apart, so the matrix core and the VALU are both kept busy; phases are
+//   separated by workgroup barriers (two per step).
+// * K of step j+3 and V of step j+2 are fetched from global memory into registers during the MFMA
+//   phase of step j, one 16-byte piece per slot, right after the piece fetched a step earlier has
+//   been handed to LDS; nothing is waited for at the end of a step.
+// * The int32 Q.K^T accumulators start from the bit pattern of 1.5 * 2^23, so their bits ARE the
+//   float kBias + dot and no int -> float conversion is issued; the two score register sets swap
+//   roles every step (the loop body exists for both parities).
 // * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
 //   rare steps where a row maximum jumps.
 #include <utility>
@@ -43,8 +49,13 @@ constexpr float kBias = 12582912.0f;
 // exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
 // product the bias is subtracted explicitly instead.
 constexpr float kBiasFoldLimit = 8192.0f;
-constexpr int kFastThreads = 512;  // 8 waves
-constexpr int kFastRows = 256;     // query rows per workgroup
+#ifndef SAGE_WAVES
+#define SAGE_WAVES 8
+#endif
+constexpr int kFastWaves = SAGE_WAVES;            // waves per workgroup, 32 query rows each
+constexpr int kFastThreads = 64 * kFastWaves;
+constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
+constexpr int kFastWgPerCu = 8 / kFastWaves;      // two waves per SIMD either way
 
 template <int D>
 struct FT {
@@ -70,7 +81,7 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 }
 
 template <int D, typename VT, bool CAUSAL>
-__global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
+__global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
     using F = FT<D>;
     using PVT = PV<VT>;
     using vec16 = typename PVT::vec;
@@ -109,7 +120,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         for (int t = 0; t < F::KSTEPS; t++)
             qf[t] = row_ok ? *reinterpret_cast<const v4i*>(qp + 16 * t) : v4i{0, 0, 0, 0};
     }
-    const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + min(2 * iq + (wave >> 2), a.nq - 1)];
+    const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + min((kFastRows / BM) * iq + (wave >> 2), a.nq - 1)];
     const float* ksp = a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk;
     const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
     const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
@@ -199,26 +210,16 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
 
     // ---- the step pipeline -----------------------------------------------------------------
-    // One iteration issues QK_SLOTS + PV_SLOTS matrix instructions.  Each "slot" is one MFMA plus
-    // the VALU work that runs in its shadow, fenced so that the order written here is the order
-    // issued:
-    //   E(u), u = 0..15: two scores of the CURRENT step -> exp2 -> 16-bit pair of P -> row sum
-    //   H(u), u = 0..7 : four scores of the NEXT step (whose Q.K^T finished earlier in this very
-    //                    iteration) -> fp32 -> running raw maximum
-    // LDS fragment reads are issued a few slots ahead of the MFMA that consumes them.
+    // The MFMA phase of a step issues QK_SLOTS + PV_SLOTS matrix instructions.  Each "slot" is one
+    // MFMA plus the few VALU / LDS instructions that run in its shadow, fenced so that the order
+    // written here is the order issued; LDS fragment reads are issued a few slots ahead of the
+    // MFMA that consumes them.
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int UPS = 24 / NSLOTS;  // units per slot
-#ifndef SAGE_KDIST
-#define SAGE_KDIST 4
-#endif
-#ifndef SAGE_VDIST
-#define SAGE_VDIST 3
-#endif
-    constexpr int KDIST = SAGE_KDIST < QK_SLOTS ? SAGE_KDIST : QK_SLOTS;  // K fragments in flight
-    constexpr int VDIST = SAGE_VDIST < QK_SLOTS ? SAGE_VDIST : QK_SLOTS - 1;  // V fragments in flight
-    static_assert(UPS * NSLOTS == 24 && KDIST <= QK_SLOTS && VDIST < QK_SLOTS, "slot plan");
+    constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
+    constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
+    static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
 
     // Scores live in two register sets that swap roles every step (the loop body is instantiated
     // for both parities), so the accumulators Q.K^T writes in one iteration are read in place by
@@ -275,54 +276,25 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
 #define PROF_T(v)
 #endif
 
+    // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
+    // (Q.K^T of the next step, P.V of this one, with the row sums and the next step's raw maximum
+    // in the shadow of the matrix instructions); the two waves that share a SIMD run half a step
+    // apart (see the barrier before the loop), so one feeds the matrix core while the other
+    // occupies the VALU.  Two barriers per step.
     auto body = [&](auto pc, int step) {
         constexpr int P = decltype(pc)::value;  // == step & 1
-        PROF_T(t_top);
         const unsigned char* kb_next = smem + (1 - P) * F::K_BYTES + kf_off;
         const unsigned char* vb_cur = smem + P * F::V_BYTES + vtr_off;
-        const int n0_next = (step + 1) * BN;
-        float sc_n = qs * ksp[min(step + 1, nsteps - 1)];
-        if (CAUSAL) sc_n = fmaxf(sc_n, 1.17549435e-38f);
-        const bool masked_n = CAUSAL && (n0_next + BN - 1 > m0 + 32 * wave + shift);
+        const int n0 = step * BN;
+        PROF_T(t_top);
+        (void)n0;
 
-        v4i kfr[QK_SLOTS];
-        vec16 vfr[PV_SLOTS];
-        auto read_k = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-#if defined(SAGE_ABL) && (SAGE_ABL == 10 || SAGE_ABL == 12)
-            kfr[i] = qf[(i + 1) % F::KSTEPS];
-            (void)kb_next;
-#else
-            kfr[i] = *reinterpret_cast<const v4i*>(kb_next + 32 * (i / F::KSTEPS) * F::K_RS + 16 * (i % F::KSTEPS));
-#endif
-        };
-        auto read_v = [&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const unsigned char* p0 = vb_cur + 16 * (j / F::DTILES) * F::V_RS + 64 * (j % F::DTILES);
-#if defined(SAGE_ABL) && (SAGE_ABL == 10 || SAGE_ABL == 12)
-            vfr[j] = __builtin_bit_cast(vec16, qf[j % F::KSTEPS]);
-            (void)p0;
-#elif defined(SAGE_ABL) && SAGE_ABL == 13
-            {
-                typedef int v2i __attribute__((ext_vector_type(2)));
-                const v2i lo = *reinterpret_cast<const v2i*>(p0), hi = *reinterpret_cast<const v2i*>(p0 + 8 * F::V_RS);
-                const v4i both = {lo[0], lo[1], hi[0], hi[1]};
-                vfr[j] = __builtin_bit_cast(vec16, both);
-            }
-#elif defined(SAGE_ABL) && SAGE_ABL == 14
-            vfr[j] = *reinterpret_cast<const vec16*>(smem + F::V_BASE + P * F::V_BYTES + (lane & 31) * 272 + (lane >> 5) * 16 + (j % 8) * 32 + (j / 8) * 8704);
-            (void)p0;
-#else
-            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
-#endif
-        };
-        sfor<KDIST>(read_k);
-        __builtin_amdgcn_sched_barrier(0);
-
-        // ---- finish the row maximum of this step; advance the running maximum only on a jump
+        // ===== VALU phase: exponentials of this step (scores in sbuf[P]; their raw maximum was
+        //       taken in the shadow of the previous MFMA phase) =====
+        const float rmx = raw_max;
         {
-            const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, raw_max),
-                                                            __builtin_bit_cast(unsigned, raw_max), false, false);
+            const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, rmx),
+                                                            __builtin_bit_cast(unsigned, rmx), false, false);
             const float rmax = (fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) - kBias) * sc;
             const float m_new = fmaxf(m_i, rmax);
             if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
@@ -335,10 +307,10 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
                     for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
             }
         }
-        float neg_m;  // exponent of a score with biased bits x: fma(x, sc, neg_m)
+        float neg_m;
         if (kBias * sc < kBiasFoldLimit) {
             neg_m = __builtin_fmaf(-kBias, sc, -m_i);
-        } else {  // large block scales: remove the bias first (exact), keep full precision
+        } else {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -350,11 +322,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
         }
         vec16 pf[4];
         float lsum = 0.0f;
-        float raw_max_n = -INFINITY;
-        __builtin_amdgcn_sched_barrier(0);
-        PROF_T(t_head);
-
-        auto exp_unit = [&](auto uc) {
+        sfor<16>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
             const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
@@ -362,63 +330,69 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
             const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc, neg_m));
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
-            lsum = PVT::dot2_ones(pf[tp], w, lsum);
-            asm volatile("" ::"v"(lsum));  // pin to this slot
-        };
-        auto slots = [&](auto maskc) {
-            constexpr bool MASKED = decltype(maskc)::value != 0;
-            sfor<NSLOTS>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-#ifdef SAGE_PRIO
-                // The two waves that share a SIMD trade issue priority halfway through the step so
-                // that they reach the barrier together.
-                if constexpr (i == 0) {
-                    if (wave < 4) __builtin_amdgcn_s_setprio(SAGE_PRIO); else __builtin_amdgcn_s_setprio(0);
-                }
-                if constexpr (i == NSLOTS / 2) {
-                    if (wave < 4) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(SAGE_PRIO);
-                }
-#endif
-                if constexpr (i < QK_SLOTS) {
-                    constexpr int kt = i / F::KSTEPS, t = i % F::KSTEPS;
-                    if constexpr (t == 0) {
-                        sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], bias16, 0, 0, 0);
-                    } else {
-                        sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
-                    }
-                    if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
-                    if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
-                } else {
-                    constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
-                    o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
-                    if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
-                    // K of step+2 and V of step+1 were fetched into registers during the previous
-                    // iteration: hand one piece per slot to LDS (those buffers were released by the
-                    // barrier that ended it) and refill the register with the tile after it.  Neither
-                    // the fetch nor the LDS write is waited for at the end of a step.
-                    if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, min(step + 3, nsteps - 1));
-                    else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, min(step + 2, nsteps - 1));
-                }
-                sfor<UPS>([&](auto rc) {
-                    constexpr int u = i * UPS + decltype(rc)::value;
-                    if constexpr (u < 16) exp_unit(IC<u>{});
-                    else head_unit(IC<1 - P>{}, IC<u - 16>{}, n0_next, MASKED, raw_max_n);
-                });
-                __builtin_amdgcn_sched_barrier(0);
-            });
-        };
-        if (CAUSAL && masked_n) slots(IC<1>{});
-        else slots(IC<0>{});
+        });
+        sc = qs * ksp[min(step + 1, nsteps - 1)];
+        if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
+        __builtin_amdgcn_sched_barrier(0);
+        PROF_T(t_head);
+        __syncthreads();  // phase switch: this wave takes the matrix core
+        PROF_T(t_slots);
 
+        // ===== MFMA phase =====
+        __builtin_amdgcn_s_setprio(1);
+        float raw_max_n = -INFINITY;
+        const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > m0 + 32 * wave + shift);
+        v4i kfr[QK_SLOTS];
+        vec16 vfr[PV_SLOTS];
+        auto read_k = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            kfr[i] = *reinterpret_cast<const v4i*>(kb_next + 32 * (i % 2) * F::K_RS + 16 * (i / 2));
+        };
+        auto read_v = [&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const unsigned char* p0 = vb_cur + 16 * (j / F::DTILES) * F::V_RS + 64 * (j % F::DTILES);
+            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+        };
+        sfor<KDIST>(read_k);
+        sfor<NSLOTS>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if constexpr (i < QK_SLOTS) {
+                constexpr int kt = i % 2, t = i / 2;  // alternate the two accumulation chains
+                if constexpr (t == 0) {
+                    sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], bias16, 0, 0, 0);
+                } else {
+                    sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
+                }
+                if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
+                if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
+                // row sums of P ride in the shadow of the Q.K^T instructions
+                sfor<16 / QK_SLOTS>([&](auto rc) {
+                    constexpr int u = i * (16 / QK_SLOTS) + decltype(rc)::value;
+                    lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
+                    asm volatile("" ::"v"(lsum));
+                });
+            } else {
+                constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
+                o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
+                if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
+                if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, min(step + 3, nsteps - 1));
+                else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, min(step + 2, nsteps - 1));
+                // raw maximum of the next step's scores (Q.K^T finished above) under the P.V instructions
+                sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
+                    constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
+                    if constexpr (u < 8) {
+                        if (CAUSAL && masked_n) head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, true, raw_max_n);
+                        else head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, false, raw_max_n);
+                    }
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
         l_i += lsum;
         raw_max = raw_max_n;
-        sc = sc_n;
-        __builtin_amdgcn_sched_barrier(0);  // the fetched tiles are only waited for after the math of this step
-        PROF_T(t_slots);
+        __builtin_amdgcn_s_setprio(0);
         PROF_T(t_store);
-#if !(defined(SAGE_ABL) && (SAGE_ABL == 3 || SAGE_ABL == 12))
-        __syncthreads();
-#endif
+        __syncthreads();  // phase switch: this wave goes back to the VALU
 #ifdef SAGE_PROF
         {
             PROF_T(t_end);
@@ -427,11 +401,13 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
 #endif
     };
 
+    if (wave >= kFastWaves / 2) __syncthreads();  // second half of the waves runs one phase behind
     for (int step = 0; step < nsteps; step += 2) {
         body(IC<0>{}, step);
         if (step + 1 >= nsteps) break;
         body(IC<1>{}, step + 1);
     }
+    if (wave < kFastWaves / 2) __syncthreads();
 
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
     const float l_o = __shfl_xor(l_i, 32);
@@ -465,7 +441,7 @@ __global__ __launch_bounds__(kFastThreads, 1) void sage_attn_fwd_fast_kernel(Att
     }
 #ifdef SAGE_PROF
     if (a.lse && lane == 0) {  // debug build: per-wave cycle totals of the loop phases replace the lse output
-        float* dst = a.lse + ((int64_t)blockIdx.x * 8 + wave) * 4;
+        float* dst = a.lse + ((int64_t)blockIdx.x * kFastWaves + wave) * 4;
         for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
     }
 #endif
