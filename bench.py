@@ -105,6 +105,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="after the timed region, run 3 device-to-device tensor copies of this many MiB "
+                         "(known traffic, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every (batch, head, q-block) is independent; "
@@ -226,6 +229,13 @@ def main():
                            "frac": round(quant_bytes / (quant_med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                            "algorithmic_bytes_per_step": quant_bytes},
     }
+    if args.calibration_copy_mib > 0:
+        src = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)  # one read + one write of known size under its own kernel name
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes"] = int(src.numel())
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(name, q, k, v)
     print(json.dumps(result))

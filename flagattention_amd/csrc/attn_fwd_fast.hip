@@ -163,17 +163,18 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         }
     };
     // piecewise variants used inside the step pipeline (one 16-byte piece per call)
-    auto restage_k = [&](auto jc, int buf, int tile) {
+    // (uniform 64-bit tile pointer + unsigned 32-bit lane offset: one scalar-base load instruction)
+    auto restage_k = [&](auto jc, int buf, const unsigned char* tile) {
         constexpr int j = decltype(jc)::value;
         if (F::K_ITEMS >= kFastThreads || k_worker) {
             *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
-            kreg[j] = *reinterpret_cast<const v4i*>(kg + (int64_t)tile * BN * a.ks_n + k_goff[j]);
+            kreg[j] = *reinterpret_cast<const v4i*>(tile + (unsigned)k_goff[j]);
         }
     };
-    auto restage_v = [&](auto ic, int buf, int tile) {
+    auto restage_v = [&](auto ic, int buf, const unsigned char* tile) {
         constexpr int i = decltype(ic)::value;
         *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
-        vreg[i] = *reinterpret_cast<const v4i*>(vg + (int64_t)tile * BN * a.vs_n + v_goff[i]);
+        vreg[i] = *reinterpret_cast<const v4i*>(tile + 2u * (unsigned)v_goff[i]);
     };
     auto store_v = [&](int buf) {
 #pragma unroll
@@ -190,7 +191,11 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // accumulator bits reinterpreted as fp32 ARE kBias + dot, so no int -> float conversion is needed.
     v16i bias16;
 #pragma unroll
-    for (int i = 0; i < 16; i++) bias16[i] = kBiasBits;
+    for (int i = 0; i < 16; i++) {
+        int b;  // materialised once through an opaque move, so the block stays in VGPRs for the whole kernel
+        asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "s"(kBiasBits));
+        bias16[i] = b;
+    }
     auto qk_tile = [&](const unsigned char* kbase, int kt) {
         v16i acc = bias16;
 #pragma unroll
@@ -275,6 +280,11 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 #else
 #define PROF_T(v)
 #endif
+
+    // tiles fetched during step 0 (K of step 3, V of step 2, clamped to the last step)
+    const int64_t k_tile_bytes = (int64_t)BN * a.ks_n, v_tile_bytes = (int64_t)BN * a.vs_n * 2;
+    const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg) + min(3, nsteps - 1) * k_tile_bytes;
+    const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg) + min(2, nsteps - 1) * v_tile_bytes;
 
     // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
     // (Q.K^T of the next step, P.V of this one, with the row sums and the next step's raw maximum
@@ -375,8 +385,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                 o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
                 if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
-                if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, min(step + 3, nsteps - 1));
-                else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, min(step + 2, nsteps - 1));
+                if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, k_fetch);
+                else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, v_fetch);
                 // raw maximum of the next step's scores (Q.K^T finished above) under the P.V instructions
                 sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
                     constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
@@ -390,6 +400,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         });
         l_i += lsum;
         raw_max = raw_max_n;
+        if (step + 4 < nsteps) k_fetch += k_tile_bytes;  // next iteration fetches K of step+4, V of step+3
+        if (step + 3 < nsteps) v_fetch += v_tile_bytes;
         __builtin_amdgcn_s_setprio(0);
         PROF_T(t_store);
         __syncthreads();  // phase switch: this wave goes back to the VALU
