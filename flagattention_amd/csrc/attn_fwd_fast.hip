@@ -340,6 +340,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc, neg_m));
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
+#ifdef SAGE_DOT2_IN_VALU_PHASE
+            lsum = PVT::dot2_ones(pf[tp], w, lsum);
+#endif
         });
         sc = qs * ksp[min(step + 1, nsteps - 1)];
         if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
@@ -349,7 +352,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         PROF_T(t_slots);
 
         // ===== MFMA phase =====
+#ifndef SAGE_NOPRIO
         __builtin_amdgcn_s_setprio(1);
+#endif
         float raw_max_n = -INFINITY;
         const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > m0 + 32 * wave + shift);
         v4i kfr[QK_SLOTS];
@@ -376,11 +381,13 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
                 if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
                 // row sums of P ride in the shadow of the Q.K^T instructions
+#ifndef SAGE_DOT2_IN_VALU_PHASE
                 sfor<16 / QK_SLOTS>([&](auto rc) {
                     constexpr int u = i * (16 / QK_SLOTS) + decltype(rc)::value;
                     lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
                     asm volatile("" ::"v"(lsum));
                 });
+#endif
             } else {
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                 o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
@@ -402,7 +409,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         raw_max = raw_max_n;
         if (step + 4 < nsteps) k_fetch += k_tile_bytes;  // next iteration fetches K of step+4, V of step+3
         if (step + 3 < nsteps) v_fetch += v_tile_bytes;
+#ifndef SAGE_NOPRIO
         __builtin_amdgcn_s_setprio(0);
+#endif
         PROF_T(t_store);
         __syncthreads();  // phase switch: this wave goes back to the VALU
 #ifdef SAGE_PROF

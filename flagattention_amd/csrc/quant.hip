@@ -247,7 +247,15 @@ __global__ __launch_bounds__(kThreads) void k_mean_final_kernel(KMeanArgs a, int
     const int d = (int)(ch % a.D);
     const float* p = a.part + bh * a.nchunk * a.D + d;
     float tot = 0.0f;
-    for (int c = 0; c < a.nchunk; c++) tot = tot + p[(int64_t)c * a.D];
+    int c = 0;
+    for (; c + 8 <= a.nchunk; c += 8) {  // loads issued together, additions kept in chunk order
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = p[(int64_t)(c + i) * a.D];
+#pragma unroll
+        for (int i = 0; i < 8; i++) tot = tot + v[i];
+    }
+    for (; c < a.nchunk; c++) tot = tot + p[(int64_t)c * a.D];
     const float mean = tot / (float)a.N;
     if (a.out_dt == SAGE_F32) static_cast<float*>(a.out)[ch] = mean;
     else if (a.out_dt == SAGE_BF16) static_cast<__bf16*>(a.out)[ch] = (__bf16)mean;
