@@ -33,6 +33,10 @@ PEAK_INT8_TOPS = 5000.0
 PEAK_16BIT_TFLOPS = 2500.0
 PEAK_MIXED_TOPS = 1.0 / (0.5 / PEAK_INT8_TOPS + 0.5 / PEAK_16BIT_TFLOPS)  # 3333.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per attention launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch, scaled by the factors a 256 MiB read+write kernel gives in the same run: 2.00 / 1.00);
+# summaries under profiles/.  None = not measured for that workload.
+MEASURED_ATTN_TRAFFIC_BYTES = {"c2": 402.9e6}
 
 WORKLOADS = {
     # name: (B, H, N, D, dtype, layout, causal, description)
@@ -219,7 +223,9 @@ def main():
             "peak": round(PEAK_MIXED_TOPS, 1),
             "unit": "TFLOP/s",
             "frac": round(attn_tops / PEAK_MIXED_TOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(name),
+            "traffic_unit": "bytes per launch (offline rocprofv3 counters, see profiles/)",
+            "algorithmic_bytes_per_launch": numel * (1 + 1 + esz) + numel * out_dtype.itemsize,
             "peak_note": "mixed dense-MFMA roofline: half the ops INT8 at 5000 TOP/s, half 16-bit at 2500 TFLOP/s",
             "algorithmic_ops_per_launch": ops,
             "avg_launch_ms": round(attn_avg, 4),

@@ -222,8 +222,14 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
-    constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
+#ifndef SAGE_KDIST
+#define SAGE_KDIST 4
+#endif
+#ifndef SAGE_VDIST
+#define SAGE_VDIST 3
+#endif
+    constexpr int KDIST = SAGE_KDIST < QK_SLOTS ? SAGE_KDIST : QK_SLOTS;      // K fragments in flight
+    constexpr int VDIST = SAGE_VDIST < QK_SLOTS ? SAGE_VDIST : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
 
     // Scores live in two register sets that swap roles every step (the loop body is instantiated
