@@ -57,19 +57,31 @@ constexpr int kFastThreads = 64 * kFastWaves;
 constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
 constexpr int kFastWgPerCu = 8 / kFastWaves;      // two waves per SIMD either way
 
+// LDS tiles are unpadded ([64 keys][row bytes]) because they are filled by direct-to-LDS loads, which
+// write 1 KB per wave instruction contiguously; bank conflicts are avoided by XOR-swizzling the
+// 16-byte chunk index of every row (the swizzle is applied on the global-address side of the load
+// and undone by the fragment reads).
 template <int D>
 struct FT {
     static constexpr int KSTEPS = D / 32;
     static constexpr int DTILES = D / 32;
-    static constexpr int K_RS = D + 16;       // bytes per K row in LDS
+    static constexpr int K_RS = D;            // bytes per K row in LDS (int8)
     static constexpr int K_BYTES = BN * K_RS;
-    static constexpr int V_RS = 2 * D + 64;   // bytes per V row in LDS
+    static constexpr int V_RS = 2 * D;        // bytes per V row in LDS (16-bit)
     static constexpr int V_BYTES = BN * V_RS;
-    static constexpr int K_ITEMS = BN * (D / 16);  // 16-byte pieces per K tile
-    static constexpr int K_LOADS = (K_ITEMS + kFastThreads - 1) / kFastThreads;
-    static constexpr int V_LOADS = BN * (D / 8) / kFastThreads;
-    static constexpr int V_BASE = 2 * K_BYTES;
-    static constexpr int TOTAL = 2 * K_BYTES + 2 * V_BYTES;
+    static constexpr int KCPR = K_RS / 16;    // 16-byte chunks per K row
+    static constexpr int VCPR = V_RS / 16;
+    static constexpr int K_INSTR = K_BYTES / 1024;  // wave-level 1 KB loads per K tile (8 | 4)
+    static constexpr int V_INSTR = V_BYTES / 1024;  // (16 | 8)
+    static constexpr int NBUF = 3;            // tiles of K (and of V) resident in LDS
+    static constexpr int V_BASE = NBUF * K_BYTES;
+    static constexpr int TOTAL = NBUF * (K_BYTES + V_BYTES);
+    static constexpr int NK = K_INSTR >= kFastWaves ? K_INSTR / kFastWaves : 1;  // loads per wave per tile
+    static constexpr int NV = V_INSTR / kFastWaves;
+    // K: 16 lanes read the same chunk of 16 consecutive rows; 256 bytes of banks hold 16 / KCPR rows
+    static __device__ __forceinline__ int k_swz(int row) { return (row / (16 / KCPR)) & (KCPR - 1); }
+    // V (transposed reads touch rows 4h + s, s = 0..3, 64 bytes each): spread s over the 64-byte windows
+    static __device__ __forceinline__ int v_swz(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
 };
 
 template <typename VT>
@@ -87,6 +99,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     using vec16 = typename PVT::vec;
     __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
 
+#ifdef SAGE_PROF
+    const long long t_kernel0 = __builtin_readcyclecounter();
+#endif
+#ifdef SAGE_PROF2
+    const long long t_k0 = __builtin_readcyclecounter();
+#endif
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -121,71 +139,67 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             qf[t] = row_ok ? *reinterpret_cast<const v4i*>(qp + 16 * t) : v4i{0, 0, 0, 0};
     }
     const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + min((kFastRows / BM) * iq + (wave >> 2), a.nq - 1)];
-    const float* ksp = a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk;
+    // k_scale is read through the constant address space: the loads stay scalar (s_load_dword) even though
+    // the loop contains assembly that clobbers memory, and they are tracked by lgkmcnt, not by the vmcnt
+    // the direct-to-LDS loads are tracked with
+    typedef __attribute__((address_space(4))) const float* const_f32_ptr;
+    const const_f32_ptr ksp = (const_f32_ptr)(uintptr_t)(a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk);
     const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
     const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
 
-    // staging: 16-byte pieces, consecutive lanes along a row
-    int k_goff[F::K_LOADS], k_lds[F::K_LOADS], v_goff[F::V_LOADS], v_lds[F::V_LOADS];
-    const bool k_worker = tid < F::K_ITEMS;
-#pragma unroll
-    for (int j = 0; j < F::K_LOADS; j++) {
-        const int id = (tid + kFastThreads * j) % F::K_ITEMS;
-        const int row = id / (D / 16), c = id % (D / 16);
-        k_goff[j] = row * (int)a.ks_n + 16 * c;
-        k_lds[j] = row * F::K_RS + 16 * c;
+    // ---- staging: direct-to-LDS loads, 16 bytes per lane, 1 KB per wave instruction.  LDS piece
+    //      p = 64 * instr + lane is chunk p % CPR of row p / CPR and receives the chunk (p % CPR) ^ swz(row)
+    //      of that row from global memory.  Wave w issues instructions w, w + 8, ... of a tile (a K tile of
+    //      head_dim 64 has only four, which waves 4-7 load a second time so that every wave has the same
+    //      number of loads in flight).  The swizzle of a wave's piece does not depend on which of its
+    //      instructions carries it (rows advance by a multiple of the swizzle period), so one per-lane
+    //      byte offset serves all of them and the instruction index only moves the uniform base.
+    static_assert(kFastWaves == 8 && F::V_INSTR % kFastWaves == 0, "load split");
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int k_idx = wave_u % F::K_INSTR;
+    unsigned k_goff, v_goff;
+    {
+        const int pk = 64 * k_idx + lane, rk = pk / F::KCPR;
+        k_goff = rk * (int)a.ks_n + 16 * ((pk % F::KCPR) ^ F::k_swz(rk));
+        const int pv = 64 * wave_u + lane, rv = pv / F::VCPR;
+        v_goff = rv * (int)a.vs_n * 2 + 16 * ((pv % F::VCPR) ^ F::v_swz(rv));
     }
-#pragma unroll
-    for (int i = 0; i < F::V_LOADS; i++) {
-        const int id = tid + kFastThreads * i;
-        const int row = id / (D / 8), c = id % (D / 8);
-        v_goff[i] = row * (int)a.vs_n + 8 * c;
-        v_lds[i] = F::V_BASE + row * F::V_RS + 16 * c;
-    }
-    v4i kreg[F::K_LOADS];
-    v4i vreg[F::V_LOADS];  // native vectors: a struct type here ends up as a stack array in LDS
-    auto load_k = [&](int tile) {
-        const int8_t* kt = kg + (int64_t)tile * BN * a.ks_n;
-        if (F::K_ITEMS >= kFastThreads || k_worker) {
-#pragma unroll
-            for (int j = 0; j < F::K_LOADS; j++) kreg[j] = *reinterpret_cast<const v4i*>(kt + k_goff[j]);
+    static_assert((64 * kFastWaves / F::KCPR) % (16 / F::KCPR * F::KCPR) == 0 && (64 * kFastWaves / F::VCPR) % 4 == 0, "swizzle period");
+    const int64_t k_instr_bytes = (int64_t)(64 * kFastWaves / F::KCPR) * a.ks_n;      // rows per round of the waves * row stride
+    const int64_t v_instr_bytes = (int64_t)(64 * kFastWaves / F::VCPR) * a.vs_n * 2;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+    // The loads are written in assembly: the compiler would otherwise wait for every outstanding one
+    // before each LDS read that follows.  Completion is tracked by hand with s_waitcnt vmcnt.
+    auto dma16 = [](const unsigned char* base, unsigned voff, unsigned lds_addr) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
+    };
+    // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions
+    auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int vbuf, const unsigned char* vtile) {
+        constexpr int e = decltype(ec)::value;
+        if constexpr (e < F::NK) {
+            dma16(ktile + e * k_instr_bytes, k_goff, lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
+        } else {
+            constexpr int ev = e - F::NK;
+            dma16(vtile + ev * v_instr_bytes, v_goff, lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
     };
-    auto load_v = [&](int tile) {
-        const VT* vt = vg + (int64_t)tile * BN * a.vs_n;
-#pragma unroll
-        for (int i = 0; i < F::V_LOADS; i++) vreg[i] = *reinterpret_cast<const v4i*>(vt + v_goff[i]);
-    };
-    auto store_k = [&](int buf) {
-        if (F::K_ITEMS >= kFastThreads || k_worker) {
-#pragma unroll
-            for (int j = 0; j < F::K_LOADS; j++) *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
-        }
-    };
-    // piecewise variants used inside the step pipeline (one 16-byte piece per call)
-    // (uniform 64-bit tile pointer + unsigned 32-bit lane offset: one scalar-base load instruction)
-    auto restage_k = [&](auto jc, int buf, const unsigned char* tile) {
-        constexpr int j = decltype(jc)::value;
-        if (F::K_ITEMS >= kFastThreads || k_worker) {
-            *reinterpret_cast<v4i*>(smem + buf * F::K_BYTES + k_lds[j]) = kreg[j];
-            kreg[j] = *reinterpret_cast<const v4i*>(tile + (unsigned)k_goff[j]);
-        }
-    };
-    auto restage_v = [&](auto ic, int buf, const unsigned char* tile) {
-        constexpr int i = decltype(ic)::value;
-        *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
-        vreg[i] = *reinterpret_cast<const v4i*>(tile + 2u * (unsigned)v_goff[i]);
-    };
-    auto store_v = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < F::V_LOADS; i++) *reinterpret_cast<v4i*>(smem + buf * F::V_BYTES + v_lds[i]) = vreg[i];
-    };
+    constexpr int NDMA = F::NK + F::NV;  // loads per wave per step
 
-    // fragment read offsets
-    const int kf_off = l32 * F::K_RS + 16 * half * (D / 32);
-    // ds_read_b64_tr_b16: in each group of 16 lanes, lane 4s+a supplies keys row s, channels 4a..4a+3,
+    // ---- fragment read offsets (undoing the swizzle)
+    // K: lane (row l32, half) reads chunk half * D/32 + t of its row for k-step t
+    int kf_off[F::KSTEPS];
+#pragma unroll
+    for (int t = 0; t < F::KSTEPS; t++) kf_off[t] = l32 * F::K_RS + 16 * ((half * (D / 32) + t) ^ F::k_swz(l32));
+    // V, ds_read_b64_tr_b16: in each group of 16 lanes, lane 4s+a supplies keys row s, channels 4a..4a+3,
     // and lane i receives channel i of the four rows.  Groups: (channels 0-15 | 16-31) x (half 0 | 1).
-    const int vtr_off = F::V_BASE + (4 * half + ((lane >> 2) & 3)) * F::V_RS + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    int vtr_off[F::DTILES];
+    {
+        const int s4 = (lane >> 2) & 3, a4 = lane & 3, g1 = (lane >> 4) & 1;
+#pragma unroll
+        for (int dt = 0; dt < F::DTILES; dt++)
+            vtr_off[dt] = (4 * half + s4) * F::V_RS + 16 * ((4 * dt + 2 * g1 + (a4 >> 1)) ^ F::v_swz(s4)) + 8 * (a4 & 1);
+    }
 
     // The int32 accumulators start from the bit pattern of the float 1.5 * 2^23: since |dot| < 2^22,
     // accumulator bits reinterpreted as fp32 ARE kBias + dot, so no int -> float conversion is needed.
@@ -200,7 +214,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         v16i acc = bias16;
 #pragma unroll
         for (int t = 0; t < F::KSTEPS; t++) {
-            const v4i kf = *reinterpret_cast<const v4i*>(kbase + kf_off + 32 * kt * F::K_RS + 16 * t);
+            const v4i kf = *reinterpret_cast<const v4i*>(kbase + kf_off[t] + 32 * kt * F::K_RS);
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[t], acc, 0, 0, 0);
         }
         return acc;
@@ -260,16 +274,20 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         asm volatile("" ::"v"(acc));  // pin to this slot (otherwise sunk below the matrix instructions)
     };
 
-    // ---- prologue: K0, V0, K1 in LDS; scores of step 0 in registers
-    load_k(0);
-    load_v(0);
-    store_k(0);
-    store_v(0);
-    load_k(min(1, nsteps - 1));
-    store_k(1);
+    // ---- prologue: K0, K1, K2, V0, V1 in LDS; scores of step 0 in registers.  Tile indices past the
+    //      last step are clamped to it: such a tile is fetched again into a buffer nobody reads.
+    const int64_t k_tile_bytes = (int64_t)BN * a.ks_n, v_tile_bytes = (int64_t)BN * a.vs_n * 2;
+    const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg);
+    const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg);
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, 0, k_fetch, 0, v_fetch); });
+    if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; }
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, 1, k_fetch, 1, v_fetch); });
+    if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; }
+    sfor<F::NK>([&](auto ec) { dma_unit(ec, 2, k_fetch, 2, v_fetch); });
+    // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
+    if (nsteps > 3) k_fetch += k_tile_bytes;
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
-    load_k(min(2, nsteps - 1));  // stored to LDS at the top of the first iteration
-    load_v(min(1, nsteps - 1));
     sbuf[0][0] = qk_tile(smem, 0);
     sbuf[0][1] = qk_tile(smem, 1);
     raw_max = -INFINITY;
@@ -282,26 +300,37 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 
 #ifdef SAGE_PROF
     long long prof[4] = {0, 0, 0, 0};
+    const long long t_loop0 = __builtin_readcyclecounter();
 #define PROF_T(v) const long long v = __builtin_readcyclecounter(); asm volatile("" ::: "memory")
+#elif defined(SAGE_FENCES)
+#define PROF_T(v) asm volatile("" ::: "memory")
 #else
 #define PROF_T(v)
 #endif
-
-    // tiles fetched during step 0 (K of step 3, V of step 2, clamped to the last step)
-    const int64_t k_tile_bytes = (int64_t)BN * a.ks_n, v_tile_bytes = (int64_t)BN * a.vs_n * 2;
-    const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg) + min(3, nsteps - 1) * k_tile_bytes;
-    const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg) + min(2, nsteps - 1) * v_tile_bytes;
 
     // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
     // (Q.K^T of the next step, P.V of this one, with the row sums and the next step's raw maximum
     // in the shadow of the matrix instructions); the two waves that share a SIMD run half a step
     // apart (see the barrier before the loop), so one feeds the matrix core while the other
     // occupies the VALU.  Two barriers per step.
-    auto body = [&](auto pc, int step) {
-        constexpr int P = decltype(pc)::value;  // == step & 1
-        const unsigned char* kb_next = smem + (1 - P) * F::K_BYTES + kf_off;
-        const unsigned char* vb_cur = smem + P * F::V_BYTES + vtr_off;
+    auto body = [&](auto pc, int step, int c3) {
+        constexpr int P = decltype(pc)::value;  // == step & 1; c3 == step % 3
+        // tile t of K (of V) lives in LDS buffer t % 3: this step reads K of step+1 and V of step, and
+        // fetches K of step+3 (into the buffer of K of step) and V of step+2
+        const int c3n = c3 == 2 ? 0 : c3 + 1, c3p = c3 == 0 ? 2 : c3 - 1;
+        int kaddr[F::KSTEPS], vaddr[F::DTILES];
+#pragma unroll
+        for (int t = 0; t < F::KSTEPS; t++) {
+            kaddr[t] = kf_off[t] + c3n * F::K_BYTES;
+            asm volatile("" : "+v"(kaddr[t]));  // computed once per step, here in the VALU phase
+        }
+#pragma unroll
+        for (int dt = 0; dt < F::DTILES; dt++) {
+            vaddr[dt] = vtr_off[dt] + F::V_BASE + c3 * F::V_BYTES;
+            asm volatile("" : "+v"(vaddr[dt]));
+        }
         const int n0 = step * BN;
+        const bool live = step < nsteps;  // false only for the padding step after an odd number of steps
         PROF_T(t_top);
         (void)n0;
 
@@ -312,7 +341,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, rmx),
                                                             __builtin_bit_cast(unsigned, rmx), false, false);
             const float rmax = (fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) - kBias) * sc;
-            const float m_new = fmaxf(m_i, rmax);
+            const float m_new = live ? fmaxf(m_i, rmax) : m_i;
             if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
                 const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
                 l_i *= alpha;
@@ -336,6 +365,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 }
             neg_m = -m_i;
         }
+        if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
         vec16 pf[4];
         float lsum = 0.0f;
         sfor<16>([&](auto uc) {
@@ -354,7 +384,26 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
         __builtin_amdgcn_sched_barrier(0);
         PROF_T(t_head);
-        __syncthreads();  // phase switch: this wave takes the matrix core
+        // The first K fragments of the coming MFMA phase are requested before the barrier (their tile
+        // landed a step ago), so the phase does not open with an LDS round trip.
+        v4i kfr[QK_SLOTS];
+        vec16 vfr[PV_SLOTS];
+        auto read_k = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            kfr[i] = *reinterpret_cast<const v4i*>(smem + kaddr[i / 2] + 32 * (i % 2) * F::K_RS);
+        };
+        auto read_v = [&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const unsigned char* p0 = smem + vaddr[j % F::DTILES] + 16 * (j / F::DTILES) * F::V_RS;
+            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+        };
+        sfor<KDIST>(read_k);
+        __builtin_amdgcn_sched_barrier(0);
+        // The direct-to-LDS loads this wave issued in its previous MFMA phase have landed (vmcnt(0)): the
+        // tiles they belong to are first read two barriers from here.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();        // phase switch: this wave takes the matrix core
+        __builtin_amdgcn_sched_barrier(0);
         PROF_T(t_slots);
 
         // ===== MFMA phase =====
@@ -363,18 +412,6 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 #endif
         float raw_max_n = -INFINITY;
         const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > m0 + 32 * wave + shift);
-        v4i kfr[QK_SLOTS];
-        vec16 vfr[PV_SLOTS];
-        auto read_k = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            kfr[i] = *reinterpret_cast<const v4i*>(kb_next + 32 * (i % 2) * F::K_RS + 16 * (i / 2));
-        };
-        auto read_v = [&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const unsigned char* p0 = vb_cur + 16 * (j / F::DTILES) * F::V_RS + 64 * (j % F::DTILES);
-            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
-        };
-        sfor<KDIST>(read_k);
         sfor<NSLOTS>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if constexpr (i < QK_SLOTS) {
@@ -385,6 +422,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                     sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
                 }
                 if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
+                if constexpr (i < NDMA) dma_unit(ic, c3, k_fetch, c3p, v_fetch);
                 if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
                 // row sums of P ride in the shadow of the Q.K^T instructions
 #ifndef SAGE_DOT2_IN_VALU_PHASE
@@ -398,8 +436,6 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                 o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
                 if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
-                if constexpr (j < F::K_LOADS) restage_k(IC<j>{}, P, k_fetch);
-                else if constexpr (j < F::K_LOADS + F::V_LOADS) restage_v(IC<j - F::K_LOADS>{}, 1 - P, v_fetch);
                 // raw maximum of the next step's scores (Q.K^T finished above) under the P.V instructions
                 sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
                     constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
@@ -419,7 +455,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         __builtin_amdgcn_s_setprio(0);
 #endif
         PROF_T(t_store);
-        __syncthreads();  // phase switch: this wave goes back to the VALU
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
+        __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
+        __builtin_amdgcn_sched_barrier(0);
 #ifdef SAGE_PROF
         {
             PROF_T(t_end);
@@ -429,47 +467,91 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     };
 
     if (wave >= kFastWaves / 2) __syncthreads();  // second half of the waves runs one phase behind
-    for (int step = 0; step < nsteps; step += 2) {
-        body(IC<0>{}, step);
-        if (step + 1 >= nsteps) break;
-        body(IC<1>{}, step + 1);
+    // The loop always runs an even number of steps (no exit between the two parities: the accumulators
+    // then stay in one set of registers); after an odd nsteps the extra step multiplies V by P = 0.
+    for (int step = 0, c3 = 0; step < nsteps; step += 2) {
+        body(IC<0>{}, step, c3);
+        body(IC<1>{}, step + 1, c3 == 2 ? 0 : c3 + 1);
+        c3 = c3 == 0 ? 2 : c3 - 1;  // (c3 + 2) % 3
     }
+    PROF_T(t_loop1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // every direct-to-LDS load of this wave has landed
+    PROF_T(t_dma_done);
     if (wave < kFastWaves / 2) __syncthreads();
+    __syncthreads();  // nobody reads or fills a K/V tile any more: the LDS is free for the output
 
+    PROF_T(t_epi0);
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
     const float l_o = __shfl_xor(l_i, 32);
     const float l_tot = half ? (l_o + l_i) : (l_i + l_o);
     const float inv = 1.0f / l_tot;
-    if (row_ok) {
-        const int64_t obase = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)my_m * a.os_n;
+    const int64_t obase_wave = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)(m0 + 32 * wave) * a.os_n;
+    if (a.out_dt != SAGE_F32) {
+        // 16-bit outputs: a lane holds its row in 8-byte pieces, which stored directly would scatter 32
+        // partial lines per instruction.  Each wave transposes its 32 rows through its own slice of LDS
+        // and writes whole rows, 16 bytes per lane.
+        constexpr int ORS = 2 * D + 16;  // bytes per staged row
+        static_assert(kFastWaves * 32 * ORS <= F::TOTAL, "output staging fits in the tile buffers");
+        unsigned char* mine = smem + wave * 32 * ORS;
+#pragma unroll
+        for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float r[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] = o[dt][4 * g + i] * inv;
+                s16x4 w;
+                if (a.out_dt == SAGE_BF16) {
+                    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+                    w = __builtin_bit_cast(s16x4, b4{(__bf16)r[0], (__bf16)r[1], (__bf16)r[2], (__bf16)r[3]});
+                } else {
+                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                    w = __builtin_bit_cast(s16x4, h4{(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]});
+                }
+                *reinterpret_cast<s16x4*>(mine + l32 * ORS + 2 * (32 * dt + 8 * g + 4 * half)) = w;
+            }
+        asm volatile("" ::: "memory");  // the reads below see other lanes' writes (same wave: LDS keeps program order)
+        constexpr int LPR = 2 * D / 16, RPI = 64 / LPR;  // lanes per row, rows per wave instruction
+        unsigned char* outp = reinterpret_cast<unsigned char*>(a.out) + 2 * obase_wave + 16 * (lane % LPR);
+#pragma unroll
+        for (int e = 0; e < 32 / RPI; e++) {
+            const int r = RPI * e + lane / LPR;
+            const v4i piece = *reinterpret_cast<const v4i*>(mine + r * ORS + 16 * (lane % LPR));
+            if (m0 + 32 * wave + r < a.M) *reinterpret_cast<v4i*>(outp + 2 * (int64_t)r * a.os_n) = piece;
+        }
+    } else if (row_ok) {
+        float* outp = static_cast<float*>(a.out) + obase_wave + (int64_t)l32 * a.os_n;
 #pragma unroll
         for (int dt = 0; dt < F::DTILES; dt++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d = 32 * dt + 8 * g + 4 * half;
-                float r[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) r[i] = o[dt][4 * g + i] * inv;
-                if (a.out_dt == SAGE_BF16) {
-                    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
-                    b4 w = {(__bf16)r[0], (__bf16)r[1], (__bf16)r[2], (__bf16)r[3]};
-                    *reinterpret_cast<b4*>(static_cast<__bf16*>(a.out) + obase + d) = w;
-                } else if (a.out_dt == SAGE_F16) {
-                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-                    h4 w = {(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
-                    *reinterpret_cast<h4*>(static_cast<_Float16*>(a.out) + obase + d) = w;
-                } else {
-                    *reinterpret_cast<v4f*>(static_cast<float*>(a.out) + obase + d) = v4f{r[0], r[1], r[2], r[3]};
-                }
+                *reinterpret_cast<v4f*>(outp + d) = v4f{o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv, o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv};
             }
-#ifndef SAGE_PROF
+    }
+    if (row_ok) {
+#if !defined(SAGE_PROF) && !defined(SAGE_PROF2)
         if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
 #endif
     }
+#ifdef SAGE_PROF2
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (a.lse && lane == 0) a.lse[(int64_t)blockIdx.x * kFastWaves + wave] = (float)(__builtin_readcyclecounter() - t_k0);
+#endif
 #ifdef SAGE_PROF
     if (a.lse && lane == 0) {  // debug build: per-wave cycle totals of the loop phases replace the lse output
-        float* dst = a.lse + ((int64_t)blockIdx.x * kFastWaves + wave) * 4;
+        float* dst = a.lse + ((int64_t)blockIdx.x * kFastWaves + wave) * 8;
         for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
+        dst[4] = (float)(t_loop0 - t_kernel0);                       // prologue
+        PROF_T(t_issued);
+        dst[0] = (float)(t_loop1 - t_loop0); dst[1] = (float)(t_dma_done - t_loop1); dst[2] = (float)(t_epi0 - t_dma_done); dst[3] = (float)(t_issued - t_epi0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        dst[5] = (float)(__builtin_readcyclecounter() - t_kernel0);  // whole kernel, output stores included
+        dst[6] = (float)(t_kernel0 & 0xFFFFFF);                      // start time (low bits)
+        unsigned hwid; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        unsigned xcc; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        dst[7] = (float)(((xcc & 15) << 8) | ((hwid >> 8) & 0xFF));
     }
 #endif
 }
