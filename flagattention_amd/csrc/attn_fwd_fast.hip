@@ -8,22 +8,24 @@
 // products S^T = K.Q^T (8 x v_mfma_i32_32x32x32_i8) and O^T += V^T.P^T (16 x v_mfma_f32_32x32x16)
 // so that a lane owns one query row and P never leaves registers.
 //
-// * V is staged in LDS as it lies in memory ([key][channel], rows padded by 64 bytes) and read
-//   with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel: exactly
-//   the A operand of the P.V MFMA, with no shuffling instructions.
+// * K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4, 16 bytes per
+//   lane), four tiles of each resident: tile t lives in buffer t % 4 and is fetched during the VALU
+//   phase two (V) or three (K) steps before the step that multiplies with it.  LDS rows are
+//   unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks of a row, applied
+//   on the global-address side of the load and undone by the fragment reads.
+// * V is read with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel:
+//   exactly the A operand of the P.V MFMA, with no shuffling instructions.
 // * Every wave alternates between a VALU phase (exponentials of step j) and an MFMA phase (Q.K^T of
 //   step j+1 and P.V of step j back to back, with the row sums of P and the raw row maximum of
 //   step j+1 riding in the shadow of the matrix instructions).  The two waves that share a SIMD
 //   run half a step apart, so the matrix core and the VALU are both kept busy; phases are
 //   separated by workgroup barriers (two per step).
-// * K of step j+3 and V of step j+2 are fetched from global memory into registers during the MFMA
-//   phase of step j, one 16-byte piece per slot, right after the piece fetched a step earlier has
-//   been handed to LDS; nothing is waited for at the end of a step.
 // * The int32 Q.K^T accumulators start from the bit pattern of 1.5 * 2^23, so their bits ARE the
 //   float kBias + dot and no int -> float conversion is issued; the two score register sets swap
 //   roles every step (the loop body exists for both parities).
 // * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
 //   rare steps where a row maximum jumps.
+// * 16-bit outputs are transposed through LDS and written as whole rows.
 #include <utility>
 
 #include "attn_common.h"
@@ -49,10 +51,7 @@ constexpr float kBias = 12582912.0f;
 // exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
 // product the bias is subtracted explicitly instead.
 constexpr float kBiasFoldLimit = 8192.0f;
-#ifndef SAGE_WAVES
-#define SAGE_WAVES 8
-#endif
-constexpr int kFastWaves = SAGE_WAVES;            // waves per workgroup, 32 query rows each
+constexpr int kFastWaves = 8;                     // waves per workgroup, 32 query rows each
 constexpr int kFastThreads = 64 * kFastWaves;
 constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
 constexpr int kFastWgPerCu = 8 / kFastWaves;      // two waves per SIMD either way
@@ -73,7 +72,7 @@ struct FT {
     static constexpr int VCPR = V_RS / 16;
     static constexpr int K_INSTR = K_BYTES / 1024;  // wave-level 1 KB loads per K tile (8 | 4)
     static constexpr int V_INSTR = V_BYTES / 1024;  // (16 | 8)
-    static constexpr int NBUF = 3;            // tiles of K (and of V) resident in LDS
+    static constexpr int NBUF = 4;            // tiles of K (and of V) resident in LDS
     static constexpr int V_BASE = NBUF * K_BYTES;
     static constexpr int TOTAL = NBUF * (K_BYTES + V_BYTES);
     static constexpr int NK = K_INSTR >= kFastWaves ? K_INSTR / kFastWaves : 1;  // loads per wave per tile
@@ -99,12 +98,6 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     using vec16 = typename PVT::vec;
     __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
 
-#ifdef SAGE_PROF
-    const long long t_kernel0 = __builtin_readcyclecounter();
-#endif
-#ifdef SAGE_PROF2
-    const long long t_k0 = __builtin_readcyclecounter();
-#endif
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -236,14 +229,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-#ifndef SAGE_KDIST
-#define SAGE_KDIST 4
-#endif
-#ifndef SAGE_VDIST
-#define SAGE_VDIST 3
-#endif
-    constexpr int KDIST = SAGE_KDIST < QK_SLOTS ? SAGE_KDIST : QK_SLOTS;      // K fragments in flight
-    constexpr int VDIST = SAGE_VDIST < QK_SLOTS ? SAGE_VDIST : QK_SLOTS - 1;  // V fragments in flight
+    constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
+    constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
 
     // Scores live in two register sets that swap roles every step (the loop body is instantiated
@@ -298,41 +285,39 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     sc = qs * ksp[0];
     if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
 
-#ifdef SAGE_PROF
-    long long prof[4] = {0, 0, 0, 0};
-    const long long t_loop0 = __builtin_readcyclecounter();
-#define PROF_T(v) const long long v = __builtin_readcyclecounter(); asm volatile("" ::: "memory")
-#elif defined(SAGE_FENCES)
-#define PROF_T(v) asm volatile("" ::: "memory")
-#else
-#define PROF_T(v)
-#endif
-
     // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
     // (Q.K^T of the next step, P.V of this one, with the row sums and the next step's raw maximum
     // in the shadow of the matrix instructions); the two waves that share a SIMD run half a step
     // apart (see the barrier before the loop), so one feeds the matrix core while the other
     // occupies the VALU.  Two barriers per step.
-    auto body = [&](auto pc, int step, int c3) {
-        constexpr int P = decltype(pc)::value;  // == step & 1; c3 == step % 3
-        // tile t of K (of V) lives in LDS buffer t % 3: this step reads K of step+1 and V of step, and
-        // fetches K of step+3 (into the buffer of K of step) and V of step+2
-        const int c3n = c3 == 2 ? 0 : c3 + 1, c3p = c3 == 0 ? 2 : c3 - 1;
+    auto body = [&](auto pc, int step) {
+        constexpr int P = decltype(pc)::value;  // == step & 1
+        // tile t of K (of V) lives in LDS buffer t % 4: this step reads K of step+1 and V of step, and
+        // fetches K of step+3 and V of step+2 into the buffers that K of step-1 and V of step-2 left
         int kaddr[F::KSTEPS], vaddr[F::DTILES];
 #pragma unroll
         for (int t = 0; t < F::KSTEPS; t++) {
-            kaddr[t] = kf_off[t] + c3n * F::K_BYTES;
+            kaddr[t] = kf_off[t] + ((step + 1) & 3) * F::K_BYTES;
             asm volatile("" : "+v"(kaddr[t]));  // computed once per step, here in the VALU phase
         }
 #pragma unroll
         for (int dt = 0; dt < F::DTILES; dt++) {
-            vaddr[dt] = vtr_off[dt] + F::V_BASE + c3 * F::V_BYTES;
+            vaddr[dt] = vtr_off[dt] + F::V_BASE + (step & 3) * F::V_BYTES;
             asm volatile("" : "+v"(vaddr[dt]));
         }
+        v4i kfr[QK_SLOTS];
+        vec16 vfr[PV_SLOTS];
+        auto read_k = [&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            kfr[i] = *reinterpret_cast<const v4i*>(smem + kaddr[i / 2] + 32 * (i % 2) * F::K_RS);
+        };
+        auto read_v = [&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const unsigned char* p0 = smem + vaddr[j % F::DTILES] + 16 * (j / F::DTILES) * F::V_RS;
+            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
+        };
         const int n0 = step * BN;
         const bool live = step < nsteps;  // false only for the padding step after an odd number of steps
-        PROF_T(t_top);
-        (void)n0;
 
         // ===== VALU phase: exponentials of this step (scores in sbuf[P]; their raw maximum was
         //       taken in the shadow of the previous MFMA phase) =====
@@ -366,6 +351,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             neg_m = -m_i;
         }
         if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
+        // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
+        // instruction.
+        sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, (step + 2) & 3, v_fetch); });
         vec16 pf[4];
         float lsum = 0.0f;
         sfor<16>([&](auto uc) {
@@ -376,40 +364,22 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc, neg_m));
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
-#ifdef SAGE_DOT2_IN_VALU_PHASE
-            lsum = PVT::dot2_ones(pf[tp], w, lsum);
-#endif
         });
         sc = qs * ksp[min(step + 1, nsteps - 1)];
         if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
         __builtin_amdgcn_sched_barrier(0);
-        PROF_T(t_head);
         // The first K fragments of the coming MFMA phase are requested before the barrier (their tile
         // landed a step ago), so the phase does not open with an LDS round trip.
-        v4i kfr[QK_SLOTS];
-        vec16 vfr[PV_SLOTS];
-        auto read_k = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            kfr[i] = *reinterpret_cast<const v4i*>(smem + kaddr[i / 2] + 32 * (i % 2) * F::K_RS);
-        };
-        auto read_v = [&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const unsigned char* p0 = smem + vaddr[j % F::DTILES] + 16 * (j / F::DTILES) * F::V_RS;
-            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
-        };
         sfor<KDIST>(read_k);
         __builtin_amdgcn_sched_barrier(0);
-        // The direct-to-LDS loads this wave issued in its previous MFMA phase have landed (vmcnt(0)): the
+        // The loads issued in the previous VALU phase have landed (all but the NDMA just issued): the
         // tiles they belong to are first read two barriers from here.
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | NDMA);
         __builtin_amdgcn_s_barrier();        // phase switch: this wave takes the matrix core
         __builtin_amdgcn_sched_barrier(0);
-        PROF_T(t_slots);
 
         // ===== MFMA phase =====
-#ifndef SAGE_NOPRIO
         __builtin_amdgcn_s_setprio(1);
-#endif
         float raw_max_n = -INFINITY;
         const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > m0 + 32 * wave + shift);
         sfor<NSLOTS>([&](auto ic) {
@@ -422,16 +392,13 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                     sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
                 }
                 if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
-                if constexpr (i < NDMA) dma_unit(ic, c3, k_fetch, c3p, v_fetch);
                 if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
                 // row sums of P ride in the shadow of the Q.K^T instructions
-#ifndef SAGE_DOT2_IN_VALU_PHASE
                 sfor<16 / QK_SLOTS>([&](auto rc) {
                     constexpr int u = i * (16 / QK_SLOTS) + decltype(rc)::value;
                     lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
                     asm volatile("" ::"v"(lsum));
                 });
-#endif
             } else {
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                 o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
@@ -451,36 +418,22 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         raw_max = raw_max_n;
         if (step + 4 < nsteps) k_fetch += k_tile_bytes;  // next iteration fetches K of step+4, V of step+3
         if (step + 3 < nsteps) v_fetch += v_tile_bytes;
-#ifndef SAGE_NOPRIO
         __builtin_amdgcn_s_setprio(0);
-#endif
-        PROF_T(t_store);
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
         __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
         __builtin_amdgcn_sched_barrier(0);
-#ifdef SAGE_PROF
-        {
-            PROF_T(t_end);
-            prof[0] += t_head - t_top; prof[1] += t_slots - t_head; prof[2] += t_store - t_slots; prof[3] += t_end - t_store;
-        }
-#endif
     };
 
     if (wave >= kFastWaves / 2) __syncthreads();  // second half of the waves runs one phase behind
     // The loop always runs an even number of steps (no exit between the two parities: the accumulators
     // then stay in one set of registers); after an odd nsteps the extra step multiplies V by P = 0.
-    for (int step = 0, c3 = 0; step < nsteps; step += 2) {
-        body(IC<0>{}, step, c3);
-        body(IC<1>{}, step + 1, c3 == 2 ? 0 : c3 + 1);
-        c3 = c3 == 0 ? 2 : c3 - 1;  // (c3 + 2) % 3
+    for (int step = 0; step < nsteps; step += 2) {
+        body(IC<0>{}, step);
+        body(IC<1>{}, step + 1);
     }
-    PROF_T(t_loop1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // every direct-to-LDS load of this wave has landed
-    PROF_T(t_dma_done);
     if (wave < kFastWaves / 2) __syncthreads();
     __syncthreads();  // nobody reads or fills a K/V tile any more: the LDS is free for the output
-
-    PROF_T(t_epi0);
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
     const float l_o = __shfl_xor(l_i, 32);
     const float l_tot = half ? (l_o + l_i) : (l_i + l_o);
@@ -530,30 +483,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             }
     }
     if (row_ok) {
-#if !defined(SAGE_PROF) && !defined(SAGE_PROF2)
         if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
-#endif
     }
-#ifdef SAGE_PROF2
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    if (a.lse && lane == 0) a.lse[(int64_t)blockIdx.x * kFastWaves + wave] = (float)(__builtin_readcyclecounter() - t_k0);
-#endif
-#ifdef SAGE_PROF
-    if (a.lse && lane == 0) {  // debug build: per-wave cycle totals of the loop phases replace the lse output
-        float* dst = a.lse + ((int64_t)blockIdx.x * kFastWaves + wave) * 8;
-        for (int i = 0; i < 4; i++) dst[i] = (float)prof[i];
-        dst[4] = (float)(t_loop0 - t_kernel0);                       // prologue
-        PROF_T(t_issued);
-        dst[0] = (float)(t_loop1 - t_loop0); dst[1] = (float)(t_dma_done - t_loop1); dst[2] = (float)(t_epi0 - t_dma_done); dst[3] = (float)(t_issued - t_epi0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        dst[5] = (float)(__builtin_readcyclecounter() - t_kernel0);  // whole kernel, output stores included
-        dst[6] = (float)(t_kernel0 & 0xFFFFFF);                      // start time (low bits)
-        unsigned hwid; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        unsigned xcc; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        dst[7] = (float)(((xcc & 15) << 8) | ((hwid >> 8) & 0xFF));
-    }
-#endif
 }
 
 template <int D, typename VT>
