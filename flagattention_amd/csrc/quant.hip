@@ -74,8 +74,8 @@ __device__ __forceinline__ float round_to(float x, int dt) {
 }
 
 // One workgroup = one quantization block of `blk` rows; UNITS 8-element groups per thread.
-template <int DT, int UNITS>
-__global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArgs a) {
+template <int DT, int UNITS, int THREADS>
+__global__ __launch_bounds__(THREADS) void quant_per_block_int8_kernel(QuantArgs a) {
     const int tid = threadIdx.x;
     const int bid = blockIdx.x;
     const int ib = bid % a.nblk;
@@ -87,11 +87,18 @@ __global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArg
     const int64_t o_base = (int64_t)b * a.os_b + (int64_t)h * a.os_h;
     const int64_t k_base = (int64_t)b * a.ks_b + (int64_t)h * a.ks_h;
 
+    // When km is broadcast along the sequence (stride 0) and head_dim / 8 is a power of two not above
+    // the thread count, a thread keeps its channel group for all its units, so the K mean of that
+    // group is loaded once.
+    const bool fixed_c8 = a.ks_n == 0 && a.d8_shift >= 0 && a.D8 <= THREADS;
+    float m_fixed[8];
+    if (a.km && fixed_c8) load8_rt(a.km, a.km_dt, k_base + (tid & (a.D8 - 1)) * 8, m_fixed);
+
     float v[UNITS][8];
     float amax = 0.0f;
 #pragma unroll
     for (int j = 0; j < UNITS; j++) {
-        const int u = tid + kThreads * j;
+        const int u = tid + THREADS * j;
         int row, c8;
         if (a.d8_shift >= 0) {
             row = u >> a.d8_shift;
@@ -106,7 +113,12 @@ __global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArg
             load8<DT>(a.x, x_base + (int64_t)n * a.xs_n + c8 * 8, v[j]);
             if (a.km) {
                 float m[8];
-                load8_rt(a.km, a.km_dt, k_base + (int64_t)n * a.ks_n + c8 * 8, m);
+                if (fixed_c8) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) m[e] = m_fixed[e];
+                } else {
+                    load8_rt(a.km, a.km_dt, k_base + (int64_t)n * a.ks_n + c8 * 8, m);
+                }
 #pragma unroll
                 for (int e = 0; e < 8; e++) v[j][e] = round_to(v[j][e] - m[e], a.diff_dt);
             }
@@ -124,18 +136,29 @@ __global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArg
 
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-    __shared__ float wave_max[kThreads / 64];
+    __shared__ float wave_max[THREADS / 64];
     if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    amax = wave_max[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; w++) amax = fmaxf(amax, wave_max[w]);
 
     const float scale = amax / 127.0f;
     if (tid == 0) a.scale[((int64_t)b * a.H + h) * a.nblk + ib] = scale;
     const bool zero_block = !(scale > 0.0f);  // 0/0 -> NaN in the reference; its int8 conversion yields 0
 
+    // x / scale, correctly rounded, without a division per element: with r = RN(1 / scale) (one IEEE
+    // division per block), q0 = x * r is within 1.5 ulp of the quotient; one residual correction
+    // q1 = fma(fma(-q0, scale, x), r, q0) is a faithful rounding, for which the residual is exact, and a
+    // second one is then the correctly rounded quotient (Markstein's division theorem).  Scales whose
+    // reciprocal could overflow or whose significand is all ones take the hardware division instead.
+    const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
+    const bool fast_div = scale >= 0x1p-60f && scale <= 0x1p60f && (sbits & 0x7fffffu) != 0x7fffffu;
+    const float rcp = 1.0f / scale;
+
 #pragma unroll
     for (int j = 0; j < UNITS; j++) {
-        const int u = tid + kThreads * j;
+        const int u = tid + THREADS * j;
         int row, c8;
         if (a.d8_shift >= 0) {
             row = u >> a.d8_shift;
@@ -148,11 +171,23 @@ __global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArg
         if ((u < total_units) && (n < a.L)) {
             uint32_t packed[2] = {0u, 0u};
             if (!zero_block) {
+                float y[8];
+                if (fast_div) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const float x = v[j][e];
+                        const float q0 = x * rcp;
+                        const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, scale, x), rcp, q0);
+                        y[e] = __builtin_fmaf(__builtin_fmaf(-q1, scale, x), rcp, q1);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) y[e] = v[j][e] / scale;  // IEEE fp32 divide (hipcc default is correctly rounded)
+                }
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    float y = v[j][e] / scale;  // IEEE fp32 divide (hipcc default is correctly rounded)
-                    y = y + (y >= 0.0f ? 0.5f : -0.5f);
-                    const int q = (int)y;  // truncation toward zero; |y| <= 127.5
+                    const float t = y[e] + __builtin_copysignf(0.5f, y[e]);  // reference: y + 0.5 * sign(y), sign(0) = +
+                    const int q = (int)t;  // truncation toward zero; |t| <= 128
                     packed[e >> 2] |= ((uint32_t)q & 0xffu) << (8 * (e & 3));
                 }
             }
@@ -163,14 +198,15 @@ __global__ __launch_bounds__(kThreads) void quant_per_block_int8_kernel(QuantArg
 
 template <int DT>
 int launch_one(const QuantArgs& a, int64_t nblocks, hipStream_t stream) {
+    // 512 threads with few 8-element groups each keep the register footprint small (more blocks in
+    // flight per CU); small blocks use 256 threads
     const int total_units = a.blk * a.D8;
-    const int units = (total_units + kThreads - 1) / kThreads;
-    dim3 grid((unsigned)nblocks), block(kThreads);
-    if (units <= 1) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1>), grid, block, 0, stream, a);
-    else if (units <= 2) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 2>), grid, block, 0, stream, a);
-    else if (units <= 4) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 4>), grid, block, 0, stream, a);
-    else if (units <= 8) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 8>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 16>), grid, block, 0, stream, a);
+    dim3 grid((unsigned)nblocks);
+    if (total_units <= 256) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1, 256>), grid, dim3(256), 0, stream, a);
+    else if (total_units <= 512) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1, 512>), grid, dim3(512), 0, stream, a);
+    else if (total_units <= 1024) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 2, 512>), grid, dim3(512), 0, stream, a);
+    else if (total_units <= 2048) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 4, 512>), grid, dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 8, 512>), grid, dim3(512), 0, stream, a);
     return check_launch("quant_per_block_int8_kernel");
 }
 

@@ -148,3 +148,38 @@ def test_errors(gpu_device):
         per_block_int8(q, q, tensor_layout="XYZ")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         per_block_int8(q.cpu(), q.cpu())
+
+
+@pytest.mark.parametrize("d", [128, 96, 24])
+def test_km_that_varies_along_the_sequence(d, gpu_device):
+    """km is whatever broadcasts to k (quant_per_block.py:53-54): a full-shape km has a non-zero
+    sequence stride, and head dims whose 8-groups are not a power of two take the generic indexing."""
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(1, 2, 200, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(1, 2, 333, d, generator=g).to(torch.bfloat16)
+    km_full = (torch.randn(1, 2, 333, d, generator=g) * 0.3).to(torch.bfloat16)
+    km_head = km_full[:, :1, :1]  # broadcast over heads and sequence
+    for km in (km_full, km_head):
+        want = O.per_block_int8(q, k, km=km)
+        got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=km.to(gpu_device))
+        _assert_bit_exact(got, want)
+
+
+def test_extreme_scales_take_the_hardware_divide(gpu_device):
+    """Blocks whose scale is tiny, huge or has an all-ones significand leave the reciprocal shortcut."""
+    from flag_attn.sage_attention import per_block_int8
+
+    g = torch.Generator().manual_seed(22)
+    q = torch.randn(1, 4, 128, 64, generator=g)
+    k = torch.randn(1, 4, 64, 64, generator=g)
+    q[0, 0] *= 1e-30
+    q[0, 1] *= 1e30
+    k[0, 0] *= 1e-36
+    k[0, 1] *= 1e25
+    k[0, 2] = k[0, 2].clamp(-1, 1)
+    k[0, 2, 0, 0] = 127.0 * torch.tensor(0x3FFFFFFF, dtype=torch.int32).view(torch.float32).item()  # scale significand all ones
+    want = O.per_block_int8(q, k, sm_scale=1.0)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), sm_scale=1.0)
+    _assert_bit_exact(got, want)
