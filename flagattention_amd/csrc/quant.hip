@@ -229,7 +229,7 @@ bool aligned16(const void* p, int esz, int64_t s0, int64_t s1, int64_t s2) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// K mean, fixed order.  Stage 1: one thread per (chunk of 64 rows, 8 channels) adds the rows in
+// K mean, fixed order.  Stage 1: one thread per (chunk of 64 rows, 4 channels) adds the rows in
 // order.  Stage 2: one thread per channel adds the chunk partials in order, divides, rounds.
 // ---------------------------------------------------------------------------------------------
 struct KMeanArgs {
@@ -241,39 +241,81 @@ struct KMeanArgs {
     int64_t total_items;  // B*H*nchunk*D8
 };
 
-template <int DT>
+// W consecutive channels of one row as fp32 (W = 8, 4 or 2; 16-bit inputs load 2 * W bytes)
+template <int DT, int W>
+__device__ __forceinline__ void loadw(const void* base, int64_t elem_off, float (&v)[W]) {
+    if constexpr (W == 8) {
+        load8<DT>(base, elem_off, v);
+    } else if constexpr (DT == SAGE_F32) {
+        const float* p = static_cast<const float*>(base) + elem_off;
+        if constexpr (W == 4) {
+            const float4 r = *reinterpret_cast<const float4*>(p);
+            v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+        } else {
+            const float2 r = *reinterpret_cast<const float2*>(p);
+            v[0] = r.x; v[1] = r.y;
+        }
+    } else {
+        const uint16_t* p = static_cast<const uint16_t*>(base) + elem_off;
+        uint32_t w[W / 2];
+        if constexpr (W == 4) {
+            const uint2 r = *reinterpret_cast<const uint2*>(p);
+            w[0] = r.x; w[1] = r.y;
+        } else {
+            w[0] = *reinterpret_cast<const uint32_t*>(p);
+        }
+#pragma unroll
+        for (int i = 0; i < W / 2; i++) {
+            if constexpr (DT == SAGE_BF16) {
+                v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+                v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+            } else {
+                v[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xffffu));
+                v[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+            }
+        }
+    }
+}
+
+// One thread per (chunk of 64 rows, W channels): narrow W means more threads in flight for the same
+// bytes; a wave still reads whole contiguous row segments (64 * W elements).
+template <int DT, int W>
 __global__ __launch_bounds__(kThreads) void k_mean_partial_kernel(KMeanArgs a) {
     const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (item >= a.total_items) return;
-    const int c8 = (int)(item % a.D8);
-    const int64_t t = item / a.D8;
+    const int dw = a.D / W;
+    const int cw = (int)(item % dw);
+    const int64_t t = item / dw;
     const int chunk = (int)(t % a.nchunk);
     const int64_t bh = t / a.nchunk;
     const int h = (int)(bh % a.H);
     const int64_t b = bh / a.H;
-    const int64_t base = b * a.s_b + (int64_t)h * a.s_h + c8 * 8;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int64_t base = b * a.s_b + (int64_t)h * a.s_h + cw * W;
+    float acc[W];
+#pragma unroll
+    for (int e = 0; e < W; e++) acc[e] = 0.0f;
     const int n0 = chunk * 64;
     const int rows = min(64, a.N - n0);
     int r = 0;
-    for (; r + 8 <= rows; r += 8) {
-        float v[8][8];
+    constexpr int kBatch = 16;  // rows whose loads are in flight together
+    for (; r + kBatch <= rows; r += kBatch) {
+        float v[kBatch][W];
 #pragma unroll
-        for (int i = 0; i < 8; i++) load8<DT>(a.k, base + (int64_t)(n0 + r + i) * a.s_n, v[i]);
+        for (int i = 0; i < kBatch; i++) loadw<DT, W>(a.k, base + (int64_t)(n0 + r + i) * a.s_n, v[i]);
 #pragma unroll
-        for (int i = 0; i < 8; i++)
+        for (int i = 0; i < kBatch; i++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) acc[e] = acc[e] + v[i][e];
+            for (int e = 0; e < W; e++) acc[e] = acc[e] + v[i][e];
     }
     for (; r < rows; r++) {
-        float v[8];
-        load8<DT>(a.k, base + (int64_t)(n0 + r) * a.s_n, v);
+        float v[W];
+        loadw<DT, W>(a.k, base + (int64_t)(n0 + r) * a.s_n, v);
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] = acc[e] + v[e];
+        for (int e = 0; e < W; e++) acc[e] = acc[e] + v[e];
     }
-    float4* dst = reinterpret_cast<float4*>(a.part + (bh * a.nchunk + chunk) * a.D + c8 * 8);
-    dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    float* dst = a.part + (bh * a.nchunk + chunk) * a.D + cw * W;
+#pragma unroll
+    for (int e = 0; e < W; e++) dst[e] = acc[e];
 }
 
 __global__ __launch_bounds__(kThreads) void k_mean_final_kernel(KMeanArgs a, int64_t channels) {
@@ -356,16 +398,17 @@ int launch_kmean(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype,
     a.s_b = k.stride_b; a.s_h = k.stride_h; a.s_n = k.stride_n;
     a.H = (int)H; a.N = (int)N; a.D = (int)D; a.D8 = (int)(D / 8); a.nchunk = (int)((N + 63) / 64);
     a.out_dt = out_dtype;
-    a.total_items = B * H * a.nchunk * a.D8;
+    constexpr int W = 4;  // channels per thread: 8-byte loads of 16-bit inputs, twice the threads of 16-byte loads
+    a.total_items = B * H * a.nchunk * (D / W);
     const int64_t g1 = (a.total_items + kThreads - 1) / kThreads;
     const int64_t channels = B * H * D;
     const int64_t g2 = (channels + kThreads - 1) / kThreads;
     if (g1 > 0x7fffffffLL) return fail(SAGE_E_UNSUPPORTED, "sage_k_mean: too many chunks");
     dim3 block(kThreads);
     switch (k_dtype) {
-        case SAGE_F16: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_F16>, dim3((unsigned)g1), block, 0, stream, a); break;
-        case SAGE_BF16: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_BF16>, dim3((unsigned)g1), block, 0, stream, a); break;
-        default: hipLaunchKernelGGL(k_mean_partial_kernel<SAGE_F32>, dim3((unsigned)g1), block, 0, stream, a); break;
+        case SAGE_F16: hipLaunchKernelGGL((k_mean_partial_kernel<SAGE_F16, W>), dim3((unsigned)g1), block, 0, stream, a); break;
+        case SAGE_BF16: hipLaunchKernelGGL((k_mean_partial_kernel<SAGE_BF16, W>), dim3((unsigned)g1), block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((k_mean_partial_kernel<SAGE_F32, W>), dim3((unsigned)g1), block, 0, stream, a); break;
     }
     int rc = check_launch("k_mean_partial_kernel");
     if (rc) return rc;
