@@ -85,3 +85,26 @@ def test_product_does_not_import_the_oracle():
                 if f.endswith((".py", ".hip", ".cpp", ".h")):
                     text = open(os.path.join(dirpath, f)).read()
                     assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_upstream_vendor_package_resolves_to_this_build():
+    """Apply the reference registry's rule (flag_attn/runtime/backend/op_registry.py:20-41) to the
+    shipped ``_amd`` package: absolute module names are imported as they are, the symbol is a getattr."""
+    import importlib
+    import importlib.util
+
+    import flagattention_amd
+    from flagattention_amd import sage_attention as sa
+
+    path = os.path.join(os.path.dirname(flagattention_amd.__file__), "upstream_vendor", "_amd", "__init__.py")
+    spec = importlib.util.spec_from_file_location("flag_attn_backend_amd_under_test", path)
+    backend = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(backend)
+    exports = vars(backend)["_OPERATOR_EXPORTS"]
+    assert set(exports) == {"sage_attention", "sage_attention_forward", "sage_attention_per_block_int8"}
+    assert backend.device.vendor_name == "amd" and backend.device.name == "cuda"
+    for name, (module, symbol) in exports.items():
+        assert not module.startswith("."), "absolute module names only: the package holds no kernels itself"
+        fn = getattr(importlib.import_module(module), symbol)
+        want = sa.per_block_int8 if name.endswith("per_block_int8") else sa.forward
+        assert fn is want
