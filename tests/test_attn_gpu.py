@@ -154,6 +154,39 @@ def test_uniform_v_and_zero_scale_block(gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("zero_blocks", [(0,), (3,), (1, 2, 5)])
+@pytest.mark.parametrize("m,n", [(384, 384), (256, 512)])
+def test_causal_with_zero_scale_blocks_and_odd_step_counts(zero_blocks, m, n, gpu_device):
+    """All-zero K blocks (scale 0) on and off the causal diagonal: hidden keys of such a block must
+    stay hidden (their score is 0 * anything, not exp2(0)); q-blocks that run an odd number of
+    64-key steps exercise the padding step of the pipelined kernel."""
+    q8, qs, k8, ks, v = _quantized(11, 1, 2, 1, m, n, 128, torch.bfloat16)
+    ks2 = ks.clone()
+    for j in zero_blocks:
+        ks2[..., j] = 0.0
+    o, lse = _run(gpu_device, q8, qs, k8, ks2, v, causal=True, return_lse=True, output_dtype=torch.bfloat16)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks2, causal=True)
+    assert bool(torch.isfinite(o.float()).all())
+    _gate(o, expected)
+    # The keys of a zero-scale block all score exactly 0, so their P values are one number and its
+    # rounding to bf16 (<= 2^-9 relative) no longer averages out in the row sum, which is taken over
+    # the rounded P: lse may be off by up to log2(1 + 2^-9) * (share of those keys) ~ 3e-3.
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("n", [64, 192, 320])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_odd_step_counts_and_output_dtypes(n, out_dtype, gpu_device):
+    """kv_len / 64 odd (padding step), every output dtype (16-bit outputs leave through LDS), and a
+    query length that leaves the last workgroup partly empty."""
+    q8, qs, k8, ks, v = _quantized(12, 2, 4, 2, 300, n, 64, torch.float16)
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, return_lse=True, output_dtype=out_dtype)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks)
+    assert o.dtype == out_dtype
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
+
+
 def _gpu_dequant_reference(q8, k8, v, qs, ks, heads, causal=False):
     """fp32 softmax attention of the dequantized operands for a few (batch, head) pairs, on the GPU
     (the same closed form as the oracle's attention_dequant; used where the CPU would take minutes)."""
