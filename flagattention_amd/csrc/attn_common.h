@@ -37,6 +37,7 @@ struct AttnArgs {
     int32_t Hq, Hkv, M, N, nq, nk, groups;
     int32_t out_dt, causal;
     int32_t total_wg;
+    int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
 };
 
 template <typename VT> struct PV;

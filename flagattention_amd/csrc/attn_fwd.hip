@@ -206,8 +206,28 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
 #pragma unroll
         for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
 
+    // Mask entries of a step are fetched one step ahead, like the K/V tiles, wherever a run of four
+    // keys can be read with one load (contiguous, aligned mask rows; runs that reach past kv_len are
+    // read entry by entry when they are used).
+    const int64_t mrow = MODE >= MODE_MASK_BOOL ? (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)my_m * a.ms_m : 0;
+    uint32_t mw_cur[8], mw_nxt[8];
+    float4 mf_cur[8], mf_nxt[8];
+    auto run_start = [&](int step, int r) { return step * BN + 32 * (r >> 2) + 8 * (r & 3) + 4 * half; };
+    auto load_mask = [&](int step, uint32_t (&mw)[8], float4 (&mf)[8]) {
+        if (MODE < MODE_MASK_BOOL || !a.mask_vec || !row_ok) return;
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            const int nb = run_start(step, r);
+            if (nb + 3 < a.N) {
+                if (MODE == MODE_MASK_BOOL) mw[r] = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(a.mask) + mrow + nb);
+                else mf[r] = *reinterpret_cast<const float4*>(static_cast<const float*>(a.mask) + mrow + nb);
+            }
+        }
+    };
+
     if (nsteps > 0) {
         load_tile(0);
+        load_mask(0, mw_cur, mf_cur);
         store_tile(0);
     }
     __syncthreads();
@@ -215,7 +235,10 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
     for (int step = 0; step < nsteps; step++) {
         const int buf = step & 1;
         const bool more = step + 1 < nsteps;
-        if (more) load_tile(step + 1);
+        if (more) {
+            load_tile(step + 1);
+            load_mask(step + 1, mw_nxt, mf_nxt);
+        }
         const unsigned char* base = smem + buf * T::STAGE;
         const int n0 = step * BN;
 
@@ -223,25 +246,52 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
         float madd[2][16];
         bool skip = false;
         if (MODE >= MODE_MASK_BOOL) {
-            const int64_t mrow = (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)my_m * a.ms_m;
             int any = 0;
+            // one entry: visibility / additive value of key n for this lane's row (mv: the loaded mask entry)
+            auto entry = [&](int kt, int i, int n, bool inb, bool mb, float mf, bool track) {
+                bool keep = inb;
+                if (a.causal) keep = keep && (n <= my_m + (a.N - a.M));
+                if (MODE == MODE_MASK_BOOL) {
+                    keep = keep && mb;
+                    madd[kt][i] = keep ? 0.0f : kMasked;
+                } else {
+                    float add = inb ? mf : kMasked;
+                    if (a.causal && inb && !keep) add += kMasked;
+                    madd[kt][i] = add;
+                }
+                if (track) any |= keep;  // feeds the tile-skip vote (bool masks and causal only)
+            };
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
-                    const bool inb = row_ok && n < a.N;
-                    bool keep = inb;
-                    if (a.causal) keep = keep && (n <= my_m + (a.N - a.M));
-                    if (MODE == MODE_MASK_BOOL) {
-                        if (keep) keep = static_cast<const uint8_t*>(a.mask)[mrow + (int64_t)n * a.ms_n] != 0;
-                        madd[kt][i] = keep ? 0.0f : kMasked;
-                        any |= keep;
+                for (int g = 0; g < 4; g++) {
+                    // the lane's keys come in runs of four consecutive ones
+                    const int nb = n0 + 32 * kt + 8 * g + 4 * half;
+                    if (a.mask_vec && row_ok && nb + 3 < a.N) {
+                        if (MODE == MODE_MASK_BOOL) {
+                            const uint32_t w = mw_cur[4 * kt + g];
+                            if (!a.causal) any |= (w != 0u);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) entry(kt, 4 * g + e, nb + e, true, ((w >> (8 * e)) & 0xffu) != 0, 0.0f, a.causal != 0);
+                        } else {
+                            const float4 w = mf_cur[4 * kt + g];
+                            const float wf[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                            for (int e = 0; e < 4; e++) entry(kt, 4 * g + e, nb + e, true, false, wf[e], a.causal != 0);
+                        }
                     } else {
-                        float add = inb ? static_cast<const float*>(a.mask)[mrow + (int64_t)n * a.ms_n] : kMasked;
-                        if (a.causal && inb && !keep) add += kMasked;
-                        madd[kt][i] = add;
-                        any |= keep;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int n = nb + e;
+                            const bool inb = row_ok && n < a.N;
+                            bool mb = false;
+                            float mf = 0.0f;
+                            if (inb) {
+                                if (MODE == MODE_MASK_BOOL) mb = static_cast<const uint8_t*>(a.mask)[mrow + (int64_t)n * a.ms_n] != 0;
+                                else mf = static_cast<const float*>(a.mask)[mrow + (int64_t)n * a.ms_n];
+                            }
+                            entry(kt, 4 * g + e, n, inb, mb, mf, true);
+                        }
                     }
                 }
             if (MODE == MODE_MASK_BOOL || a.causal) skip = !__syncthreads_or(any);
@@ -282,10 +332,11 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
                 for (int kt = 0; kt < 2; kt++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
-                        float x = (float)sacc[kt][i] * sc;
+                        float x;
                         if (MODE >= MODE_MASK_BOOL) {
-                            x += madd[kt][i];
+                            x = __builtin_fmaf((float)sacc[kt][i], sc, madd[kt][i]);
                         } else {
+                            x = (float)sacc[kt][i] * sc;
                             const int n = n0 + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
                             bool keep = n < a.N;
                             if (MODE == MODE_CAUSAL) keep = keep && (n <= my_m + (a.N - a.M));
@@ -346,6 +397,13 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
         }
 
         if (more) store_tile(buf ^ 1);
+        if (MODE == MODE_MASK_BOOL) {
+#pragma unroll
+            for (int r = 0; r < 8; r++) mw_cur[r] = mw_nxt[r];
+        } else if (MODE == MODE_MASK_F32) {
+#pragma unroll
+            for (int r = 0; r < 8; r++) mf_cur[r] = mf_nxt[r];
+        }
         __syncthreads();
     }
 
@@ -405,6 +463,11 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     a.nq = (int)((p.qo_len + BM - 1) / BM); a.nk = (int)((p.kv_len + BN - 1) / BN);
     a.groups = (int)(p.heads_q / p.heads_kv);
     a.out_dt = p.out_dtype; a.causal = p.causal ? 1 : 0;
+    if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_n == 1) {
+        const int64_t align = p.mask_kind == SAGE_MASK_BOOL ? 4 : 16, esz = p.mask_kind == SAGE_MASK_BOOL ? 1 : 4;
+        a.mask_vec = ((uintptr_t)p.mask % align) == 0 && (p.mask_stride_b * esz) % align == 0 &&
+                     (p.mask_stride_h * esz) % align == 0 && (p.mask_stride_m * esz) % align == 0;
+    }
     const int64_t total = p.batch * p.heads_q * a.nq;
     if (total > 0x7fffffffLL || p.qo_len > 0x7fffffffLL - BM || p.kv_len > 0x7fffffffLL - BN)
         return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: problem too large for 32-bit tile indices");

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // before each LDS read that follows.  Completion is tracked by hand with s_waitcnt vmcnt.
     auto dma16 = [](const unsigned char* base, unsigned voff, unsigned lds_addr) {
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
+                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");  // (m0 cannot be named as a clobber; nothing else in this kernel uses it)
     };
     // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions
     auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int vbuf, const unsigned char* vtile) {
