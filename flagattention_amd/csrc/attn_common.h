@@ -68,8 +68,8 @@ template <> struct PV<_Float16> {
 };
 
 
-// Launches the software-pipelined kernel for the common case (no mask tensor, kv_len a multiple
-// of 64, and qo_len <= kv_len when causal).  head_dim 64 / 128, V dtype fp16 / bf16.
+// Launches the software-pipelined kernel: no mask tensor, and qo_len <= kv_len when causal.
+// head_dim 64 / 128, V dtype fp16 / bf16.
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream);
 
 }  // namespace attn

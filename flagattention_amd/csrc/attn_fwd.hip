@@ -479,7 +479,7 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
     else if (p.mask_kind == SAGE_MASK_F32) mode = MODE_MASK_F32;
     else if (p.causal) mode = MODE_CAUSAL;
-    const bool fast = p.mask_kind == SAGE_MASK_NONE && (p.kv_len % BN) == 0 && (!p.causal || p.qo_len <= p.kv_len);
+    const bool fast = p.mask_kind == SAGE_MASK_NONE && (!p.causal || p.qo_len <= p.kv_len);
     if (fast) return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
     if (p.head_dim == 128) {
         return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)

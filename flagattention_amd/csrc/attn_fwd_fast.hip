@@ -1,5 +1,5 @@
-// Software-pipelined SageAttention forward for gfx950: the common case (no mask tensor, kv_len a
-// multiple of 64, causal only with qo_len <= kv_len).  Same arithmetic contract as the general
+// Software-pipelined SageAttention forward for gfx950: every call without a mask tensor (causal
+// only with qo_len <= kv_len; any kv_len).  Same arithmetic contract as the general
 // kernel in attn_fwd.hip (FlagAttention src/flag_attn/sage_attention/attn_qk_int8_per_block.py:
 // 20-127); what differs is how the work is laid out in time.
 //
@@ -108,17 +108,22 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     int wg = blockIdx.x;
     if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
     int iq = wg % nq2;
-    if (CAUSAL) iq = nq2 - 1 - iq;  // longest rows first
+    if (CAUSAL && a.causal) iq = nq2 - 1 - iq;  // longest rows first
     const int h = (wg / nq2) % a.Hq;
     const int b = wg / (nq2 * a.Hq);
     const int hk = h / a.groups;
     const int m0 = iq * kFastRows;
     const int my_m = m0 + 32 * wave + l32;
     const bool row_ok = my_m < a.M;
-    const int shift = a.N - a.M;  // causal: key n is visible to row m iff n <= m + shift
+    // The CAUSAL instance is the one that can hide keys: key n is visible to row m iff n <= lim(m), with
+    // lim = min(m + kv_len - qo_len, kv_len - 1) under the causal flag and kv_len - 1 otherwise (a kv_len
+    // that is not a multiple of 64 leaves hidden keys in the last tile).
+    const int shift = a.N - a.M;
+    const int lim = !CAUSAL ? 0 : a.causal ? min(my_m + shift, a.N - 1) : a.N - 1;                  // this lane's row
+    const int wlim = !CAUSAL ? 0 : a.causal ? min(m0 + 32 * wave + shift, a.N - 1) : a.N - 1;      // first row of the wave
 
     int nsteps = a.nk;
-    if (CAUSAL) {
+    if (CAUSAL && a.causal) {
         const int last_row = min(m0 + kFastRows, a.M) - 1;
         nsteps = min(nsteps, (last_row + shift + BN) / BN);  // >= 1 because qo_len <= kv_len
     }
@@ -167,14 +172,36 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");  // (m0 cannot be named as a clobber; nothing else in this kernel uses it)
     };
-    // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions
-    auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int vbuf, const unsigned char* vtile) {
+    // The last tile of a kv_len that is not a multiple of 64 (CAUSAL instance only): rows past the end
+    // re-read the last valid row (finite values under hidden scores), through per-lane offsets of their own.
+    const bool ragged = CAUSAL && (a.N % BN) != 0;
+    unsigned k_goff_last[F::NK], v_goff_last[F::NV];
+    if (CAUSAL) {
+        const int last = (a.N - 1) % BN;
+#pragma unroll
+        for (int e = 0; e < F::NK; e++) {
+            const int pk = 64 * k_idx + lane, rk = pk / F::KCPR + e * (64 * kFastWaves / F::KCPR);
+            k_goff_last[e] = min(rk, last) * (int)a.ks_n + 16 * ((pk % F::KCPR) ^ F::k_swz(rk));
+        }
+#pragma unroll
+        for (int e = 0; e < F::NV; e++) {
+            const int pv = 64 * wave_u + lane, rv = pv / F::VCPR + e * (64 * kFastWaves / F::VCPR);
+            v_goff_last[e] = min(rv, last) * (int)a.vs_n * 2 + 16 * ((pv % F::VCPR) ^ F::v_swz(rv));
+        }
+    }
+    // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions.
+    // kt / vt: index of the tile behind ktile / vtile
+    auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int kt, int vbuf, const unsigned char* vtile, int vt) {
         constexpr int e = decltype(ec)::value;
         if constexpr (e < F::NK) {
-            dma16(ktile + e * k_instr_bytes, k_goff, lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
+            const bool cut = ragged && kt == a.nk - 1;
+            dma16(cut ? ktile : ktile + e * k_instr_bytes, cut ? k_goff_last[e] : k_goff,
+                  lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
         } else {
             constexpr int ev = e - F::NK;
-            dma16(vtile + ev * v_instr_bytes, v_goff, lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
+            const bool cut = ragged && vt == a.nk - 1;
+            dma16(cut ? vtile : vtile + ev * v_instr_bytes, cut ? v_goff_last[ev] : v_goff,
+                  lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
     };
     constexpr int NDMA = F::NK + F::NV;  // loads per wave per step
@@ -252,7 +279,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             if (CAUSAL && masked) {
                 const int i = i0 + e;
                 const int n = n0_next + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
-                x[e] = (n > my_m + shift) ? -INFINITY : x[e];
+                x[e] = (n > lim) ? -INFINITY : x[e];
                 sbuf[P][kt][i] = __builtin_bit_cast(int, x[e]);
             }
         }
@@ -266,20 +293,21 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const int64_t k_tile_bytes = (int64_t)BN * a.ks_n, v_tile_bytes = (int64_t)BN * a.vs_n * 2;
     const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg);
     const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg);
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 0, k_fetch, 0, v_fetch); });
-    if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; }
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 1, k_fetch, 1, v_fetch); });
-    if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; }
-    sfor<F::NK>([&](auto ec) { dma_unit(ec, 2, k_fetch, 2, v_fetch); });
+    int k_tile = 0, v_tile = 0;  // indices of the tiles behind k_fetch / v_fetch
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
+    if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
+    if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
+    sfor<F::NK>([&](auto ec) { dma_unit(ec, 2, k_fetch, k_tile, 2, v_fetch, v_tile); });
     // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
-    if (nsteps > 3) k_fetch += k_tile_bytes;
+    if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);
     sbuf[0][1] = qk_tile(smem, 1);
     raw_max = -INFINITY;
     {
-        const bool masked0 = CAUSAL && (BN - 1 > m0 + 32 * wave + shift);
+        const bool masked0 = CAUSAL && (BN - 1 > wlim);
         sfor<8>([&](auto uc) { head_unit(IC<0>{}, uc, 0, masked0, raw_max); });
     }
     sc = qs * ksp[0];
@@ -353,7 +381,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
         // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
         // instruction.
-        sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, (step + 2) & 3, v_fetch); });
+        sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
         vec16 pf[4];
         float lsum = 0.0f;
         sfor<16>([&](auto uc) {
@@ -381,7 +409,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // ===== MFMA phase =====
         __builtin_amdgcn_s_setprio(1);
         float raw_max_n = -INFINITY;
-        const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > m0 + 32 * wave + shift);
+        const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > wlim);
         sfor<NSLOTS>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if constexpr (i < QK_SLOTS) {
@@ -416,8 +444,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         });
         l_i += lsum;
         raw_max = raw_max_n;
-        if (step + 4 < nsteps) k_fetch += k_tile_bytes;  // next iteration fetches K of step+4, V of step+3
-        if (step + 3 < nsteps) v_fetch += v_tile_bytes;
+        if (step + 4 < nsteps) { k_fetch += k_tile_bytes; k_tile++; }  // next iteration fetches K of step+4, V of step+3
+        if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
         __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
@@ -501,6 +529,7 @@ int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
 }  // namespace
 
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream) {
+    causal = causal || (a.N % BN) != 0;  // the instance that can hide keys also serves a ragged last tile
     if (head_dim == 128)
         return v_dtype == SAGE_BF16 ? launch_causal<128, __bf16>(a, causal, stream)
                                     : launch_causal<128, _Float16>(a, causal, stream);

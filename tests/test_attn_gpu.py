@@ -187,6 +187,24 @@ def test_odd_step_counts_and_output_dtypes(n, out_dtype, gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n", [(5, 63), (64, 65), (257, 127), (300, 449), (30, 1027)])
+def test_ragged_kv_len_with_gqa(layout, causal, m, n, gpu_device):
+    """kv_len not a multiple of 64: the keys past the end of the last tile stay hidden, with grouped
+    heads and both layouts (causal only where every row sees a key)."""
+    if causal and m > n:
+        pytest.skip("rows without a visible key are covered by test_causal")
+    q8, qs, k8, ks, v = _quantized(13, 2, 4, 2, m, n, 128, torch.bfloat16, layout)
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, tensor_layout=layout, causal=causal, return_lse=True,
+                  output_dtype=torch.bfloat16)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, layout, causal=causal)
+    _gate(o, expected)
+    # rows that see only a handful of keys: the row sum runs over P rounded to bf16 (unit roundoff
+    # 2^-8), which does not average out over so few terms -> up to log2(1 + 2^-8) = 5.6e-3 in lse
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
+
+
 def _gpu_dequant_reference(q8, k8, v, qs, ks, heads, causal=False):
     """fp32 softmax attention of the dequantized operands for a few (batch, head) pairs, on the GPU
     (the same closed form as the oracle's attention_dequant; used where the CPU would take minutes)."""
