@@ -256,6 +256,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
+    constexpr int DEFER = D == 64 ? 8 : 0;                   // exponential units moved into the MFMA phase
     constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
     constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
@@ -384,15 +385,19 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
         vec16 pf[4];
         float lsum = 0.0f;
-        sfor<16>([&](auto uc) {
+        const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
+        auto exp_unit = [&](auto uc) {  // two scores -> two 16-bit P values
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
             const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc, neg_m));
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
-        });
+        };
+        // The last DEFER of the 16 units wait for the MFMA phase (head_dim 64: that phase has half the
+        // matrix instructions, so it takes a share of the exponentials to keep the two phases even).
+        sfor<16 - DEFER>(exp_unit);
         sc = qs * ksp[min(step + 1, nsteps - 1)];
         if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
         __builtin_amdgcn_sched_barrier(0);
@@ -422,10 +427,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
                 if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
                 // row sums of P ride in the shadow of the Q.K^T instructions
-                sfor<16 / QK_SLOTS>([&](auto rc) {
-                    constexpr int u = i * (16 / QK_SLOTS) + decltype(rc)::value;
-                    lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
-                    asm volatile("" ::"v"(lsum));
+                sfor<16 - DEFER>([&](auto rc) {
+                    constexpr int u = decltype(rc)::value;
+                    if constexpr (u * QK_SLOTS / (16 - DEFER) == i) {
+                        lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
+                        asm volatile("" ::"v"(lsum));
+                    }
                 });
             } else {
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
@@ -439,6 +446,13 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                         else head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, false, raw_max_n);
                     }
                 });
+            }
+            if constexpr (i < DEFER) {  // a deferred exponential unit and its row-sum term
+                constexpr int u = 16 - DEFER + i;
+                static_assert(DEFER == 0 || QK_SLOTS + (u >> 2) * F::DTILES > i, "P is ready before the P.V slot that multiplies with it");
+                exp_unit(IC<u>{});
+                lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
+                asm volatile("" ::"v"(lsum));
             }
             __builtin_amdgcn_sched_barrier(0);
         });
