@@ -94,11 +94,16 @@ __global__ __launch_bounds__(THREADS) void quant_per_block_int8_kernel(QuantArgs
     float m_fixed[8];
     if (a.km && fixed_c8) load8_rt(a.km, a.km_dt, k_base + (tid & (a.D8 - 1)) * 8, m_fixed);
 
-    float v[UNITS][8];
-    float amax = 0.0f;
+    // All loads of the block are issued before anything waits for one: they are unconditional (a unit
+    // past the end of the block or of the sequence re-reads a valid row and is zeroed afterwards), so
+    // that the compiler keeps them together instead of one load, one wait per unit.
+    uint4 raw16[UNITS];
+    float4 raw32[UNITS][2];
+    bool live[UNITS];
+    int64_t koff[UNITS];  // km entry of the unit when km is not one row per (batch, head) (loaded where it is used)
 #pragma unroll
     for (int j = 0; j < UNITS; j++) {
-        const int u = tid + THREADS * j;
+        const int u = min(tid + THREADS * j, total_units - 1);
         int row, c8;
         if (a.d8_shift >= 0) {
             row = u >> a.d8_shift;
@@ -108,25 +113,45 @@ __global__ __launch_bounds__(THREADS) void quant_per_block_int8_kernel(QuantArgs
             c8 = u - row * a.D8;
         }
         const int n = ib * a.blk + row;
-        const bool live = (u < total_units) && (n < a.L);
-        if (live) {
-            load8<DT>(a.x, x_base + (int64_t)n * a.xs_n + c8 * 8, v[j]);
-            if (a.km) {
-                float m[8];
-                if (fixed_c8) {
-#pragma unroll
-                    for (int e = 0; e < 8; e++) m[e] = m_fixed[e];
-                } else {
-                    load8_rt(a.km, a.km_dt, k_base + (int64_t)n * a.ks_n + c8 * 8, m);
-                }
-#pragma unroll
-                for (int e = 0; e < 8; e++) v[j][e] = round_to(v[j][e] - m[e], a.diff_dt);
-            }
-            if (a.apply_mul) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) v[j][e] = v[j][e] * a.mul;
-            }
+        live[j] = (tid + THREADS * j < total_units) && (n < a.L);
+        const int64_t nc = min(n, a.L - 1);
+        const int64_t off = x_base + nc * a.xs_n + c8 * 8;
+        if constexpr (DT == SAGE_F32) {
+            const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(a.x) + off);
+            raw32[j][0] = p[0];
+            raw32[j][1] = p[1];
         } else {
+            raw16[j] = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.x) + off);
+        }
+        koff[j] = k_base + nc * a.ks_n + c8 * 8;
+    }
+
+    float v[UNITS][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < UNITS; j++) {
+        if constexpr (DT == SAGE_F32) {
+            v[j][0] = raw32[j][0].x; v[j][1] = raw32[j][0].y; v[j][2] = raw32[j][0].z; v[j][3] = raw32[j][0].w;
+            v[j][4] = raw32[j][1].x; v[j][5] = raw32[j][1].y; v[j][6] = raw32[j][1].z; v[j][7] = raw32[j][1].w;
+        } else {
+            unpack8(raw16[j], DT, v[j]);
+        }
+        if (a.km) {
+            float m[8];
+            if (fixed_c8) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) m[e] = m_fixed[e];
+            } else {
+                load8_rt(a.km, a.km_dt, koff[j], m);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[j][e] = round_to(v[j][e] - m[e], a.diff_dt);
+        }
+        if (a.apply_mul) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[j][e] = v[j][e] * a.mul;
+        }
+        if (!live[j]) {
 #pragma unroll
             for (int e = 0; e < 8; e++) v[j][e] = 0.0f;  // rows past L are masked loads: zeros
         }
@@ -168,7 +193,7 @@ __global__ __launch_bounds__(THREADS) void quant_per_block_int8_kernel(QuantArgs
             c8 = u - row * a.D8;
         }
         const int n = ib * a.blk + row;
-        if ((u < total_units) && (n < a.L)) {
+        if (live[j]) {
             uint32_t packed[2] = {0u, 0u};
             if (!zero_block) {
                 float y[8];
@@ -198,13 +223,13 @@ __global__ __launch_bounds__(THREADS) void quant_per_block_int8_kernel(QuantArgs
 
 template <int DT>
 int launch_one(const QuantArgs& a, int64_t nblocks, hipStream_t stream) {
-    // 512 threads with few 8-element groups each keep the register footprint small (more blocks in
-    // flight per CU); small blocks use 256 threads
+    // four 16-byte loads in flight per thread wherever the block is large enough, and a register
+    // footprint that keeps eight waves per SIMD resident
     const int total_units = a.blk * a.D8;
     dim3 grid((unsigned)nblocks);
     if (total_units <= 256) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1, 256>), grid, dim3(256), 0, stream, a);
-    else if (total_units <= 512) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 1, 512>), grid, dim3(512), 0, stream, a);
-    else if (total_units <= 1024) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 2, 512>), grid, dim3(512), 0, stream, a);
+    else if (total_units <= 512) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 2, 256>), grid, dim3(256), 0, stream, a);
+    else if (total_units <= 1024) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 4, 256>), grid, dim3(256), 0, stream, a);
     else if (total_units <= 2048) hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 4, 512>), grid, dim3(512), 0, stream, a);
     else hipLaunchKernelGGL((quant_per_block_int8_kernel<DT, 8, 512>), grid, dim3(512), 0, stream, a);
     return check_launch("quant_per_block_int8_kernel");
