@@ -205,6 +205,41 @@ def test_ragged_kv_len_with_gqa(layout, causal, m, n, gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
 
 
+def _sweep_cases():
+    import random
+
+    rng = random.Random(20240607)
+    cases = []
+    for i in range(40):
+        d = rng.choice([64, 128])
+        hkv = rng.choice([1, 2, 3])
+        hq = hkv * rng.choice([1, 2, 4])
+        n = rng.choice([1, 17, 64, 100, 128, 191, 192, 256, 300, 449, 512, 777])
+        causal = rng.random() < 0.4
+        m = rng.choice([1, 31, 128, 255, 256, 257, 400, 600])
+        if causal and m > n:
+            m = rng.choice([x for x in (1, 31, 128, 255, 256, 257, 400, 600) if x <= n] or [1])
+        cases.append(dict(seed=100 + i, b=rng.choice([1, 2]), hq=hq, hkv=hkv, m=m, n=n, d=d,
+                          dtype=rng.choice([torch.float16, torch.bfloat16]), layout=rng.choice(["HND", "NHD"]),
+                          causal=causal, out_dtype=rng.choice([torch.float16, torch.bfloat16, torch.float32])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: "b{b}_hq{hq}_hkv{hkv}_m{m}_n{n}_d{d}_{layout}_c{causal}".format(
+    **{k: (int(v) if isinstance(v, bool) else v) for k, v in c.items()}))
+def test_seeded_shape_sweep(case, gpu_device):
+    """Forty seeded combinations of batch, grouped heads, ragged lengths, head dim, dtypes, layout and
+    the causal flag (no mask tensor: all of them run on the pipelined kernel)."""
+    c = case
+    q8, qs, k8, ks, v = _quantized(c["seed"], c["b"], c["hq"], c["hkv"], c["m"], c["n"], c["d"], c["dtype"], c["layout"])
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, tensor_layout=c["layout"], causal=c["causal"], return_lse=True,
+                  output_dtype=c["out_dtype"])
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, c["layout"], causal=c["causal"])
+    assert o.dtype == c["out_dtype"] and o.shape == q8.shape
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
+
+
 def _gpu_dequant_reference(q8, k8, v, qs, ks, heads, causal=False):
     """fp32 softmax attention of the dequantized operands for a few (batch, head) pairs, on the GPU
     (the same closed form as the oracle's attention_dequant; used where the CPU would take minutes)."""
