@@ -183,3 +183,47 @@ def test_extreme_scales_take_the_hardware_divide(gpu_device):
     want = O.per_block_int8(q, k, sm_scale=1.0)
     got = per_block_int8(q.to(gpu_device), k.to(gpu_device), sm_scale=1.0)
     _assert_bit_exact(got, want)
+
+
+def _quant_sweep_cases():
+    import random
+
+    rng = random.Random(777)
+    cases = []
+    for i in range(30):
+        d = rng.choice([8, 24, 64, 96, 128, 256])
+        blkq, blkk = rng.choice([(128, 64), (64, 32), (16, 16), (128, 128), (32, 64)])
+        if max(blkq, blkk) * d > 32768:
+            blkq, blkk = 64, 32
+        cases.append(dict(seed=500 + i, b=rng.choice([1, 2]), h=rng.choice([1, 3]), lq=rng.choice([1, 63, 128, 129, 300, 517]),
+                          lk=rng.choice([1, 64, 65, 200, 333]), d=d, blkq=blkq, blkk=blkk,
+                          dtype=rng.choice([torch.float16, torch.bfloat16, torch.float32]),
+                          km=rng.choice(["none", "mean16", "mean32", "full"]), layout=rng.choice(["HND", "NHD"]),
+                          sm_scale=rng.choice([None, 0.3, 1.0])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _quant_sweep_cases(), ids=lambda c: "lq{lq}_lk{lk}_d{d}_b{blkq}x{blkk}_{km}_{layout}".format(**c))
+def test_seeded_quantizer_sweep(case, gpu_device):
+    """Thirty seeded combinations of lengths, head dims (8-groups that are and are not powers of two),
+    block sizes, input dtypes, km kinds and layouts: int8 and scales bit for bit."""
+    from flag_attn.sage_attention import per_block_int8
+
+    c = case
+    g = torch.Generator().manual_seed(c["seed"])
+    q = (torch.randn(c["b"], c["h"], c["lq"], c["d"], generator=g) * 1.7).to(c["dtype"])
+    k = (torch.randn(c["b"], c["h"], c["lk"], c["d"], generator=g) + 0.5).to(c["dtype"])
+    km = None
+    if c["km"] == "mean16":
+        km = k.float().mean(dim=2, keepdim=True).to(c["dtype"])
+    elif c["km"] == "mean32":
+        km = k.float().mean(dim=2, keepdim=True)
+    elif c["km"] == "full":
+        km = (torch.randn(c["b"], c["h"], c["lk"], c["d"], generator=g) * 0.2).to(c["dtype"])
+    if c["layout"] == "NHD":
+        q, k = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+        km = None if km is None else km.transpose(1, 2).contiguous()
+    kw = dict(BLKQ=c["blkq"], BLKK=c["blkk"], sm_scale=c["sm_scale"], tensor_layout=c["layout"])
+    want = O.per_block_int8(q, k, km=km, **kw)
+    got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=_gpu(km, gpu_device), **kw)
+    _assert_bit_exact(got, want)
