@@ -354,3 +354,53 @@ def test_sageattn_wrapper_lse(gpu_device):
     cos, rel, _ = O.accuracy_metrics(o.cpu(), ref.cpu())
     assert cos >= 0.999 and rel <= 0.05
     torch.testing.assert_close(lse, torch.logsumexp(s, -1), atol=5e-2, rtol=1e-3)
+
+
+def test_side_stream_and_graph_replay(gpu_device):
+    """The library only enqueues kernels on the caller's stream (reference: launches on the current
+    torch stream, attn_qk_int8_per_block.py:176): results on a side stream equal those on the default
+    stream, and a captured graph of mean -> quantize -> attention replays to the same bits, with eager
+    work between the replays."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn(2, 4, 384, 128, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
+
+    def pipeline(qx):
+        km = sa.k_mean(k)
+        q8, qs, k8, ks = sa.per_block_int8(qx, k, km=km)
+        o, lse = sa.sage_attention(q8, k8, v, qs, ks, output_dtype=torch.bfloat16, return_lse=True, causal=True)
+        return q8, qs, k8, ks, o, lse
+
+    want = [t.clone() for t in pipeline(q)]
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = pipeline(q)
+    side.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+    static_q = q.clone()
+    with torch.cuda.stream(side):
+        pipeline(static_q)  # warm-up on the capture stream (allocator)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = pipeline(static_q)
+    for rep in range(3):
+        if rep == 1:  # other input, other expected result
+            static_q.copy_(q.flip(2))
+            expect = [t.clone() for t in pipeline(q.flip(2))]
+        elif rep == 2:
+            static_q.copy_(q)
+            expect = want
+        else:
+            expect = want
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(captured, expect):
+            assert torch.equal(a, b), f"replay {rep}"
