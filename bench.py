@@ -5,7 +5,7 @@
 
 One "step" is one pass of the hot path over one batch resident in HBM:
 K mean (fixed order) -> fused smoothing + per-block INT8 quantization of Q and K -> INT8-QK
-attention forward.  The default workload is BASELINE.json's configs[1] (B4 H32 N4096 D128 bf16
+attention forward.  The default workload is the Llama-style prefill shape (B4 H32 N4096 D128 bf16
 HND, non-causal, smooth_k on).  Prints ONE JSON line:
 
 * ``value``: effective TOPS of the whole step, 4*B*H*M*N*D (causal: visible pairs only) / step time;
