@@ -16,15 +16,17 @@
 // * V is read with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel:
 //   exactly the A operand of the P.V MFMA, with no shuffling instructions.
 // * Every wave alternates between a VALU phase (exponentials of step j) and an MFMA phase (Q.K^T of
-//   step j+1 and P.V of step j back to back, with the row sums of P and the raw row maximum of
-//   step j+1 riding in the shadow of the matrix instructions).  The two waves that share a SIMD
+//   step j+1 and P.V of step j back to back, with the row sums of P riding in the shadow of the
+//   matrix instructions).  The two waves that share a SIMD
 //   run half a step apart, so the matrix core and the VALU are both kept busy; phases are
 //   separated by workgroup barriers (two per step).
 // * The int32 Q.K^T accumulators start from the bit pattern of 1.5 * 2^23, so their bits ARE the
 //   float kBias + dot and no int -> float conversion is issued; the two score register sets swap
 //   roles every step (the loop body exists for both parities).
-// * The running maximum is advanced lazily (kTau) so the O accumulators are rescaled only on the
-//   rare steps where a row maximum jumps.
+// * No row maximum is taken per step: exponentials use the reference point the row already has
+//   (the maximum of its first tile to begin with), and a step whose row sums come out large is
+//   redone against its true maximum before any P.V instruction of it has been issued.  The row
+//   sums are needed anyway, so the common step pays nothing for the check but a compare.
 // * 16-bit outputs are transposed through LDS and written as whole rows.
 #include <utility>
 
@@ -51,6 +53,7 @@ constexpr float kBias = 12582912.0f;
 // exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
 // product the bias is subtracted explicitly instead.
 constexpr float kBiasFoldLimit = 8192.0f;
+constexpr float kSumLimit = 8192.0f;  // a lane's 32 P of one step sum to less than this, or the step is redone
 constexpr int kFastWaves = 8;                     // waves per workgroup, 32 query rows each
 constexpr int kFastThreads = 64 * kFastWaves;
 constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
@@ -240,8 +243,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         return acc;
     };
 
-    float m_i = -INFINITY;
-    float l_i = half ? 0.0f : 1.0f;  // the two halves of a row sum to the reference's initial l = 1
+    float m_i;         // reference point of the row's exponentials: set from the first tile below
+    float l_i = 0.0f;  // (the reference's initial l = 1 is multiplied by exp2(-inf) = 0 in its first step)
     v16f o[F::DTILES];
 #pragma unroll
     for (int dt = 0; dt < F::DTILES; dt++)
@@ -256,16 +259,16 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int DEFER = D == 64 ? 8 : 0;                   // exponential units moved into the MFMA phase
+    constexpr int DEFER = D == 64 ? 4 : 0;                   // exponential units moved into the MFMA phase
     constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
     constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
+    static_assert(DEFER <= QK_SLOTS, "every P of a step exists when its row sums are checked, before the first P.V");
 
     // Scores live in two register sets that swap roles every step (the loop body is instantiated
     // for both parities), so the accumulators Q.K^T writes in one iteration are read in place by
     // the exponentials of the next one.
     v16i sbuf[2][2];  // [parity][32-key tile]: int32 accumulators whose bits are the float kBias + dot
-    float raw_max;    // maximum of the current step's 32 biased scores of this lane
     float sc;         // q_scale * k_scale of the current step
 
     auto as_f = [](int bits) { return __builtin_bit_cast(float, bits); };
@@ -288,6 +291,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         acc = fmaxf(fmaxf(acc, x[2]), x[3]);
         asm volatile("" ::"v"(acc));  // pin to this slot (otherwise sunk below the matrix instructions)
     };
+    // The two lanes that share a row (l32 and l32 + 32) agree on the larger of their values.
+    auto row_pair_max = [](float x) {
+        const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
+        const unsigned mine = sw[0], other = sw[1];  // (scalar copies: bit_cast of a vector element lvalue reads element 0)
+        return fmaxf(__builtin_bit_cast(float, mine), __builtin_bit_cast(float, other));
+    };
 
     // ---- prologue: K0, K1, K2, V0, V1 in LDS; scores of step 0 in registers.  Tile indices past the
     //      last step are clamped to it: such a tile is fetched again into a buffer nobody reads.
@@ -306,17 +315,18 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);
     sbuf[0][1] = qk_tile(smem, 1);
-    raw_max = -INFINITY;
-    {
-        const bool masked0 = CAUSAL && (BN - 1 > wlim);
-        sfor<8>([&](auto uc) { head_unit(IC<0>{}, uc, 0, masked0, raw_max); });
-    }
     sc = qs * ksp[0];
     if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
+    {   // the row maximum of the first tile is the reference point the row starts from
+        float raw_max = -INFINITY;
+        const bool masked0 = CAUSAL && (BN - 1 > wlim);
+        sfor<8>([&](auto uc) { head_unit(IC<0>{}, uc, 0, masked0, raw_max); });
+        m_i = (row_pair_max(raw_max) - kBias) * sc;
+    }
 
     // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
-    // (Q.K^T of the next step, P.V of this one, with the row sums and the next step's raw maximum
-    // in the shadow of the matrix instructions); the two waves that share a SIMD run half a step
+    // (Q.K^T of the next step, P.V of this one, with the row sums in the shadow of the matrix
+    // instructions); the two waves that share a SIMD run half a step
     // apart (see the barrier before the loop), so one feeds the matrix core while the other
     // occupies the VALU.  Two barriers per step.
     auto body = [&](auto pc, int step) {
@@ -348,26 +358,14 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         const int n0 = step * BN;
         const bool live = step < nsteps;  // false only for the padding step after an odd number of steps
 
-        // ===== VALU phase: exponentials of this step (scores in sbuf[P]; their raw maximum was
-        //       taken in the shadow of the previous MFMA phase) =====
-        const float rmx = raw_max;
-        {
-            const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, rmx),
-                                                            __builtin_bit_cast(unsigned, rmx), false, false);
-            const float rmax = (fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1])) - kBias) * sc;
-            const float m_new = live ? fmaxf(m_i, rmax) : m_i;
-            if (__builtin_amdgcn_ballot_w64(m_new - m_i > kTau) != 0) {
-                const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-                l_i *= alpha;
-                m_i = m_new;
-#pragma unroll
-                for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
-            }
-        }
+        // ===== VALU phase: exponentials of this step (scores in sbuf[P]) =====
+        // No row maximum is taken: the exponentials use the reference point m_i the row already has, which
+        // any value not far below the true maximum serves equally well (the result is O / l either way).
+        // Should it make a P too large, the row sums show it before the first P.V instruction, and the step
+        // is redone against its true maximum: see redo_if_large below.
         float neg_m;
-        if (kBias * sc < kBiasFoldLimit) {
+        const bool folded = kBias * sc < kBiasFoldLimit;
+        if (folded) {
             neg_m = __builtin_fmaf(-kBias, sc, -m_i);
         } else {
 #pragma unroll
@@ -398,6 +396,38 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // The last DEFER of the 16 units wait for the MFMA phase (head_dim 64: that phase has half the
         // matrix instructions, so it takes a share of the exponentials to keep the two phases even).
         sfor<16 - DEFER>(exp_unit);
+        // A lane's 32 P of a step sum to less than kSumLimit, or the step is redone: so no P overflows the
+        // 16-bit type (nor does a sum or a product with V come near the fp32 range), and a row whose scores
+        // rise keeps its reference point within log2(kSumLimit) of its maximum.  Wave-wide decision; rare
+        // after the first steps of a row (the maximum of a row rises ever more slowly).
+        auto redo_if_large = [&]() {
+            if (__builtin_amdgcn_ballot_w64(!(lsum < kSumLimit)) != 0) {  // also taken for inf and NaN
+                float raw = -INFINITY;
+#pragma unroll
+                for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int bits = sbuf[P][kt][i];
+                        raw = fmaxf(raw, as_f(bits));
+                    }
+                const float rmax = (row_pair_max(raw) - (folded ? kBias : 0.0f)) * sc_e;
+                const float m_new = fmaxf(m_i, rmax);
+                const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+                l_i *= alpha;
+                m_i = m_new;
+#pragma unroll
+                for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+                neg_m = folded ? __builtin_fmaf(-kBias, sc_e, -m_i) : -m_i;
+                lsum = 0.0f;
+                sfor<16>([&](auto uc) {
+                    constexpr int u = decltype(uc)::value;
+                    exp_unit(uc);
+                    lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
+                });
+            }
+        };
         sc = qs * ksp[min(step + 1, nsteps - 1)];
         if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
         __builtin_amdgcn_sched_barrier(0);
@@ -413,7 +443,6 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 
         // ===== MFMA phase =====
         __builtin_amdgcn_s_setprio(1);
-        float raw_max_n = -INFINITY;
         const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > wlim);
         sfor<NSLOTS>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
@@ -436,16 +465,23 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 });
             } else {
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
+                if constexpr (j == 0) {
+                    redo_if_large();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
                 if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
-                // raw maximum of the next step's scores (Q.K^T finished above) under the P.V instructions
-                sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
-                    constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
-                    if constexpr (u < 8) {
-                        if (CAUSAL && masked_n) head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, true, raw_max_n);
-                        else head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, false, raw_max_n);
-                    }
-                });
+                // hidden keys of the next step's scores (Q.K^T finished above) are set to -inf under the
+                // P.V instructions
+                if constexpr (CAUSAL) {
+                    sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
+                        constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
+                        if constexpr (u < 8) {
+                            float unused = 0.0f;
+                            if (masked_n) head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, true, unused);
+                        }
+                    });
+                }
             }
             if constexpr (i < DEFER) {  // a deferred exponential unit and its row-sum term
                 constexpr int u = 16 - DEFER + i;
@@ -457,7 +493,6 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             __builtin_amdgcn_sched_barrier(0);
         });
         l_i += lsum;
-        raw_max = raw_max_n;
         if (step + 4 < nsteps) { k_fetch += k_tile_bytes; k_tile++; }  // next iteration fetches K of step+4, V of step+3
         if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
         __builtin_amdgcn_s_setprio(0);

@@ -174,6 +174,36 @@ def test_causal_with_zero_scale_blocks_and_odd_step_counts(zero_blocks, m, n, gp
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
 
 
+_SCALE_PATTERNS = {
+    # factor on the K scale of 64-key block j: the row maxima then move between tiles by far more than
+    # the exponent range of the 16-bit P (jump, late), or by a few units every tile (ramp)
+    "jump": lambda j: [1e-3, 1.0, 300.0, 1e-3, 30.0, 1e-3, 2000.0, 1.0][j % 8],
+    "late": lambda j: 1e-4 if j < 9 else 500.0,
+    "ramp": lambda j: 0.25 * (j + 1),
+    "fall": lambda j: 400.0 / (j + 1) ** 2,
+}
+
+
+@pytest.mark.parametrize("pattern", sorted(_SCALE_PATTERNS))
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("d,vdtype", [(128, torch.bfloat16), (128, torch.float16), (64, torch.float16), (64, torch.bfloat16)])
+def test_row_maximum_that_moves_between_tiles(pattern, causal, d, vdtype, gpu_device):
+    """The kernel takes the exponentials of a tile against the reference point the row already has and
+    starts over from the tile's true maximum when the row sums come out large: K scales that differ
+    by orders of magnitude from block to block drive it through that path (a P that overflows to
+    inf, one that merely grows, a first tile far below the rest) with a known answer."""
+    m, n = 320, 768 + 64 * (d == 64)
+    q8, qs, k8, ks, v = _quantized(31, 1, 2, 1, m, n, d, vdtype)
+    ks2 = ks.clone()
+    for j in range(ks2.shape[-1]):
+        ks2[..., j] *= _SCALE_PATTERNS[pattern](j)
+    o, lse = _run(gpu_device, q8, qs, k8, ks2, v, causal=causal, return_lse=True, output_dtype=torch.float32)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks2, causal=causal)
+    assert bool(torch.isfinite(o).all()) and bool(torch.isfinite(lse).all())
+    _gate(o, expected, pattern)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-5)
+
+
 @pytest.mark.parametrize("n", [64, 192, 320])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_odd_step_counts_and_output_dtypes(n, out_dtype, gpu_device):
