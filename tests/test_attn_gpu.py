@@ -204,6 +204,36 @@ def test_row_maximum_that_moves_between_tiles(pattern, causal, d, vdtype, gpu_de
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-5)
 
 
+@pytest.mark.parametrize("pattern", sorted(_SCALE_PATTERNS))
+@pytest.mark.parametrize("path", ["ragged", "ragged_causal", "bool_mask", "additive_mask", "causal_m_gt_n"])
+def test_row_maximum_that_moves_between_tiles_other_paths(pattern, path, gpu_device):
+    """The same K-scale patterns through a ragged last tile, through both mask kinds and through
+    causal with qo_len > kv_len (the last three run the general kernel)."""
+    m, n = (320, 700) if path.startswith("ragged") else (448, 384) if path == "causal_m_gt_n" else (200, 640)
+    q8, qs, k8, ks, v = _quantized(37, 1, 2, 2, m, n, 128, torch.bfloat16)
+    ks2 = ks.clone()
+    for j in range(ks2.shape[-1]):
+        ks2[..., j] *= _SCALE_PATTERNS[pattern](j)
+    kw, okw = {}, {}
+    if path in ("ragged_causal", "causal_m_gt_n"):
+        kw = okw = {"causal": True}
+    elif path == "bool_mask":
+        g = torch.Generator().manual_seed(5)
+        mask = torch.rand(1, 1, m, n, generator=g) > 0.3
+        mask[..., 0] = True  # no fully hidden row
+        kw, okw = {"attn_mask": mask.to(gpu_device)}, {"attn_mask": mask}
+    elif path == "additive_mask":
+        g = torch.Generator().manual_seed(6)
+        mask = torch.randn(1, 2, m, n, generator=g)
+        kw, okw = {"attn_mask": mask.to(gpu_device)}, {"attn_mask": mask}
+    o, lse = _run(gpu_device, q8, qs, k8, ks2, v, return_lse=True, output_dtype=torch.float32, **kw)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks2, **okw)
+    rows = torch.isfinite(expected).all(-1)  # causal with qo_len > kv_len: rows that see no key are NaN in the reference too
+    assert bool(torch.isfinite(o.cpu()[rows]).all())
+    _gate(o.cpu()[rows], expected[rows], f"{path}/{pattern}")
+    torch.testing.assert_close(lse.cpu()[rows], expected_lse[rows], atol=6e-3, rtol=1e-5)
+
+
 @pytest.mark.parametrize("n", [64, 192, 320])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_odd_step_counts_and_output_dtypes(n, out_dtype, gpu_device):
