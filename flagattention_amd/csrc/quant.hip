@@ -376,20 +376,7 @@ int launch_quant(const sage_quant_params& p, hipStream_t stream) {
         shift = 0;
         while ((1 << shift) < D8) shift++;
     }
-    if (p.q.ptr && p.qo_len > 0) {
-        if (!aligned16(p.q.ptr, esz, p.q.stride_b, p.q.stride_h, p.q.stride_n) ||
-            !aligned_to(8, p.q_int8.ptr, 1, p.q_int8.stride_b, p.q_int8.stride_h, p.q_int8.stride_n))
-            return fail(SAGE_E_INVALID, "sage_per_block_int8: q rows must be 16-byte aligned (8-byte for int8 output)");
-        QuantArgs a{};
-        a.x = p.q.ptr; a.km = nullptr; a.out = (int8_t*)p.q_int8.ptr; a.scale = p.q_scale;
-        a.xs_b = p.q.stride_b; a.xs_h = p.q.stride_h; a.xs_n = p.q.stride_n;
-        a.os_b = p.q_int8.stride_b; a.os_h = p.q_int8.stride_h; a.os_n = p.q_int8.stride_n;
-        a.H = (int)p.heads_q; a.L = (int)p.qo_len; a.D8 = D8; a.d8_shift = shift; a.blk = p.blkq;
-        a.nblk = (int)((p.qo_len + p.blkq - 1) / p.blkq);
-        a.apply_mul = (p.q_mul != 1.0f); a.mul = p.q_mul;
-        int rc = launch_tensor(a, p.in_dtype, p.batch * p.heads_q * a.nblk, stream);
-        if (rc) return rc;
-    }
+    // K first: a caller that has just taken the K mean finds K still in the memory-side cache.
     if (p.k.ptr && p.kv_len > 0) {
         if (!aligned16(p.k.ptr, esz, p.k.stride_b, p.k.stride_h, p.k.stride_n) ||
             !aligned_to(8, p.k_int8.ptr, 1, p.k_int8.stride_b, p.k_int8.stride_h, p.k_int8.stride_n))
@@ -408,6 +395,20 @@ int launch_quant(const sage_quant_params& p, hipStream_t stream) {
         a.nblk = (int)((p.kv_len + p.blkk - 1) / p.blkk);
         a.apply_mul = 0; a.mul = 1.0f;
         int rc = launch_tensor(a, p.in_dtype, p.batch * p.heads_kv * a.nblk, stream);
+        if (rc) return rc;
+    }
+    if (p.q.ptr && p.qo_len > 0) {
+        if (!aligned16(p.q.ptr, esz, p.q.stride_b, p.q.stride_h, p.q.stride_n) ||
+            !aligned_to(8, p.q_int8.ptr, 1, p.q_int8.stride_b, p.q_int8.stride_h, p.q_int8.stride_n))
+            return fail(SAGE_E_INVALID, "sage_per_block_int8: q rows must be 16-byte aligned (8-byte for int8 output)");
+        QuantArgs a{};
+        a.x = p.q.ptr; a.km = nullptr; a.out = (int8_t*)p.q_int8.ptr; a.scale = p.q_scale;
+        a.xs_b = p.q.stride_b; a.xs_h = p.q.stride_h; a.xs_n = p.q.stride_n;
+        a.os_b = p.q_int8.stride_b; a.os_h = p.q_int8.stride_h; a.os_n = p.q_int8.stride_n;
+        a.H = (int)p.heads_q; a.L = (int)p.qo_len; a.D8 = D8; a.d8_shift = shift; a.blk = p.blkq;
+        a.nblk = (int)((p.qo_len + p.blkq - 1) / p.blkq);
+        a.apply_mul = (p.q_mul != 1.0f); a.mul = p.q_mul;
+        int rc = launch_tensor(a, p.in_dtype, p.batch * p.heads_q * a.nblk, stream);
         if (rc) return rc;
     }
     return SAGE_OK;
