@@ -227,7 +227,7 @@ def main():
         "parity": {"int8_bit_exact": int8_exact, "scale_bit_exact": scale_exact, "cosine": cos, "max_abs_err": max_abs,
                    "checked_on": "batch 0, heads 0-1 (quantizer) / head 0 (attention) of this workload vs the CPU oracle"},
         "roofline": {
-            "kernel": "sage_attn_fwd_kernel",
+            "kernel": "sage_attn_fwd_fast_kernel",
             "bound": "mfma",
             "achieved": round(attn_tops, 2),
             "peak": round(PEAK_MIXED_TOPS, 1),
