@@ -464,3 +464,14 @@ def test_side_stream_and_graph_replay(gpu_device):
         torch.cuda.synchronize()
         for a, b in zip(captured, expect):
             assert torch.equal(a, b), f"replay {rep}"
+
+
+def test_benchmark_rows_on_a_small_shape(gpu_device):
+    """One row of the upstream-runner record, torch SDPA on the same GPU as the baseline."""
+    from flagattention_amd import benchmark_rows as R
+
+    row = R.measure((1, 2, 256, 64), torch.bfloat16, warmup_ms=1, rep_ms=5)
+    assert set(R.ROW_DEFAULTS) <= set(row)
+    assert row["error_msg"] is None and row["latency"] > 0 and row["tflops"] > 0
+    if row["base_miss_reason"] is None:
+        assert row["accuracy"] >= 0.99 and row["relative_l2"] <= 0.05 and row["speedup"] > 0

@@ -108,3 +108,26 @@ def test_upstream_vendor_package_resolves_to_this_build():
         fn = getattr(importlib.import_module(module), symbol)
         want = sa.per_block_int8 if name.endswith("per_block_int8") else sa.forward
         assert fn is want
+
+
+def test_benchmark_rows_record_format(tmp_path, monkeypatch):
+    """The record written for the upstream benchmark runner: "[INFO] " + one JSON document with the
+    runner's top-level keys, rows carrying every default field (benchmark/recording.py:37-53), non-finite
+    floats as null; without a GPU the entry point reports that and fails."""
+    import json
+
+    from flagattention_amd import benchmark_rows as R
+
+    log = tmp_path / "sub" / "rows.log"
+    row = dict(R.ROW_DEFAULTS, shape_detail=[1, 2, 256, 64], latency=0.5, latency_base=float("nan"))
+    R.emit({"level": "comprehensive", "op_name": "sage_attention", "dtype": "torch.bfloat16", "mode": "kernel", "result": [row]}, str(log))
+    R.emit({"op_name": "second"}, str(log))
+    lines = log.read_text().splitlines()
+    assert len(lines) == 2 and all(line.startswith("[INFO] ") for line in lines)
+    doc = json.loads(lines[0][len("[INFO] "):])
+    assert doc["op_name"] == "sage_attention" and doc["result"][0]["latency_base"] is None
+    assert set(R.ROW_DEFAULTS) <= set(doc["result"][0])
+    assert R.baseline_name(torch.float16) == "torch_sdpa"
+    assert R.baseline_name(torch.bfloat16) == "torch_sdpa_plus_bfloat16_cast"
+    if not torch.cuda.is_available():
+        assert R.main(["--seq-lens", "128"]) == 1
