@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsage_attention_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 SAGE_F16, SAGE_BF16, SAGE_F32 = 0, 1, 2
 MASK_NONE, MASK_BOOL, MASK_F32 = 0, 1, 2
@@ -43,9 +43,21 @@ class AttnParams(ctypes.Structure):
     ]
 
 
+class FlashParams(ctypes.Structure):
+    _fields_ = [
+        ("q", SageTensor), ("k", SageTensor), ("v", SageTensor), ("out", SageTensor),
+        ("log_normalizer", ctypes.c_void_p),
+        ("batch", c_i64), ("heads_q", c_i64), ("heads_kv", c_i64), ("qo_len", c_i64), ("kv_len", c_i64),
+        ("head_dim", c_i64),
+        ("dtype", c_i32), ("out_dtype", c_i32), ("causal", c_i32),
+        ("sm_scale", ctypes.c_float),
+    ]
+
+
 EXPORTS = (
     "sage_per_block_int8",
     "sage_attn_fwd",
+    "sage_flash_attn_fwd",
     "sage_k_mean",
     "sage_k_mean_workspace_bytes",
     "sage_hip_last_error",
@@ -75,6 +87,8 @@ def load():
     lib.sage_per_block_int8.restype = ctypes.c_int
     lib.sage_attn_fwd.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_void_p]
     lib.sage_attn_fwd.restype = ctypes.c_int
+    lib.sage_flash_attn_fwd.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p]
+    lib.sage_flash_attn_fwd.restype = ctypes.c_int
     lib.sage_k_mean_workspace_bytes.argtypes = [c_i64] * 4
     lib.sage_k_mean_workspace_bytes.restype = c_i64
     lib.sage_k_mean.argtypes = [ctypes.POINTER(SageTensor), c_i32, ctypes.c_void_p, c_i32, c_i64, c_i64, c_i64,

@@ -38,6 +38,8 @@ struct AttnArgs {
     int32_t out_dt, causal;
     int32_t total_wg;
     int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
+    float lse_mul;     // factor on the base-2 log-sum-exp on its way out (1: as is; ln 2: natural log)
+    float qk_scale;    // 16-bit Q and K only: sm_scale * log2(e), the one scale of every score (q/k point at 16-bit data)
 };
 
 template <typename VT> struct PV;
@@ -71,6 +73,9 @@ template <> struct PV<_Float16> {
 // Launches the software-pipelined kernel: no mask tensor, and qo_len <= kv_len when causal.
 // head_dim 64 / 128, V dtype fp16 / bf16.
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream);
+
+// The same kernel on 16-bit Q and K (dense attention); causal with any qo_len / kv_len.
+int launch_flash(const AttnArgs& a, int head_dim, int dtype, bool causal, hipStream_t stream);
 
 }  // namespace attn
 }  // namespace sage

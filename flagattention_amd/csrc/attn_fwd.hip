@@ -463,6 +463,7 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     a.nq = (int)((p.qo_len + BM - 1) / BM); a.nk = (int)((p.kv_len + BN - 1) / BN);
     a.groups = (int)(p.heads_q / p.heads_kv);
     a.out_dt = p.out_dtype; a.causal = p.causal ? 1 : 0;
+    a.lse_mul = 1.0f;
     if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_n == 1) {
         const int64_t align = p.mask_kind == SAGE_MASK_BOOL ? 4 : 16, esz = p.mask_kind == SAGE_MASK_BOOL ? 1 : 4;
         a.mask_vec = ((uintptr_t)p.mask % align) == 0 && (p.mask_stride_b * esz) % align == 0 &&

@@ -28,541 +28,11 @@
 //   redone against its true maximum before any P.V instruction of it has been issued.  The row
 //   sums are needed anyway, so the common step pays nothing for the check but a compare.
 // * 16-bit outputs are transposed through LDS and written as whole rows.
-#include <utility>
-
-#include "attn_common.h"
+#include "attn_fast_kernel.h"
 
 namespace sage {
 namespace attn {
 namespace {
-
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
-typedef unsigned v2u __attribute__((ext_vector_type(2)));
-
-// compile-time loops: f(IC<0>{}), f(IC<1>{}), ...
-template <int I> struct IC { static constexpr int value = I; };
-template <typename Fn, int... Is>
-__device__ __forceinline__ void sfor_impl(Fn&& f, std::integer_sequence<int, Is...>) { (f(IC<Is>{}), ...); }
-template <int N, typename Fn>
-__device__ __forceinline__ void sfor(Fn&& f) { sfor_impl(f, std::make_integer_sequence<int, N>{}); }
-
-constexpr int kBiasBits = 0x4B400000;  // 12582912.0f = 1.5 * 2^23
-constexpr float kBias = 12582912.0f;
-// exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
-// product the bias is subtracted explicitly instead.
-constexpr float kBiasFoldLimit = 8192.0f;
-constexpr float kSumLimit = 8192.0f;  // a lane's 32 P of one step sum to less than this, or the step is redone
-constexpr int kFastWaves = 8;                     // waves per workgroup, 32 query rows each
-constexpr int kFastThreads = 64 * kFastWaves;
-constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
-constexpr int kFastWgPerCu = 8 / kFastWaves;      // two waves per SIMD either way
-
-// LDS tiles are unpadded ([64 keys][row bytes]) because they are filled by direct-to-LDS loads, which
-// write 1 KB per wave instruction contiguously; bank conflicts are avoided by XOR-swizzling the
-// 16-byte chunk index of every row (the swizzle is applied on the global-address side of the load
-// and undone by the fragment reads).
-template <int D>
-struct FT {
-    static constexpr int KSTEPS = D / 32;
-    static constexpr int DTILES = D / 32;
-    static constexpr int K_RS = D;            // bytes per K row in LDS (int8)
-    static constexpr int K_BYTES = BN * K_RS;
-    static constexpr int V_RS = 2 * D;        // bytes per V row in LDS (16-bit)
-    static constexpr int V_BYTES = BN * V_RS;
-    static constexpr int KCPR = K_RS / 16;    // 16-byte chunks per K row
-    static constexpr int VCPR = V_RS / 16;
-    static constexpr int K_INSTR = K_BYTES / 1024;  // wave-level 1 KB loads per K tile (8 | 4)
-    static constexpr int V_INSTR = V_BYTES / 1024;  // (16 | 8)
-    static constexpr int NBUF = 4;            // tiles of K (and of V) resident in LDS
-    static constexpr int V_BASE = NBUF * K_BYTES;
-    static constexpr int TOTAL = NBUF * (K_BYTES + V_BYTES);
-    static constexpr int NK = K_INSTR >= kFastWaves ? K_INSTR / kFastWaves : 1;  // loads per wave per tile
-    static constexpr int NV = V_INSTR / kFastWaves;
-    // K: 16 lanes read the same chunk of 16 consecutive rows; 256 bytes of banks hold 16 / KCPR rows
-    static __device__ __forceinline__ int k_swz(int row) { return (row / (16 / KCPR)) & (KCPR - 1); }
-    // V (transposed reads touch rows 4h + s, s = 0..3, 64 bytes each): spread s over the 64-byte windows
-    static __device__ __forceinline__ int v_swz(int row) { return D == 128 ? 4 * (row & 3) : 4 * ((row >> 1) & 1); }
-};
-
-template <typename VT>
-__device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0, const unsigned char* p1) {
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p0);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p1);
-    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(typename PV<VT>::vec, both);
-}
-
-template <int D, typename VT, bool CAUSAL>
-__global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
-    using F = FT<D>;
-    using PVT = PV<VT>;
-    using vec16 = typename PVT::vec;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
-
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6;
-    const int lane = tid & 63;
-    const int l32 = lane & 31;
-    const int half = lane >> 5;
-
-    // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
-    int wg = blockIdx.x;
-    if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
-    int iq = wg % nq2;
-    if (CAUSAL && a.causal) iq = nq2 - 1 - iq;  // longest rows first
-    const int h = (wg / nq2) % a.Hq;
-    const int b = wg / (nq2 * a.Hq);
-    const int hk = h / a.groups;
-    const int m0 = iq * kFastRows;
-    const int my_m = m0 + 32 * wave + l32;
-    const bool row_ok = my_m < a.M;
-    // The CAUSAL instance is the one that can hide keys: key n is visible to row m iff n <= lim(m), with
-    // lim = min(m + kv_len - qo_len, kv_len - 1) under the causal flag and kv_len - 1 otherwise (a kv_len
-    // that is not a multiple of 64 leaves hidden keys in the last tile).
-    const int shift = a.N - a.M;
-    const int lim = !CAUSAL ? 0 : a.causal ? min(my_m + shift, a.N - 1) : a.N - 1;                  // this lane's row
-    const int wlim = !CAUSAL ? 0 : a.causal ? min(m0 + 32 * wave + shift, a.N - 1) : a.N - 1;      // first row of the wave
-
-    int nsteps = a.nk;
-    if (CAUSAL && a.causal) {
-        const int last_row = min(m0 + kFastRows, a.M) - 1;
-        nsteps = min(nsteps, (last_row + shift + BN) / BN);  // >= 1 because qo_len <= kv_len
-    }
-
-    // Q fragments: lane (row l32, half) holds channels half*D/2 + 16t .. +15 of k-step t
-    v4i qf[F::KSTEPS];
-    {
-        const int8_t* qp = a.q + (int64_t)b * a.qs_b + (int64_t)h * a.qs_h + (int64_t)my_m * a.qs_n + half * (D / 2);
-#pragma unroll
-        for (int t = 0; t < F::KSTEPS; t++)
-            qf[t] = row_ok ? *reinterpret_cast<const v4i*>(qp + 16 * t) : v4i{0, 0, 0, 0};
-    }
-    const float qs = a.q_scale[((int64_t)b * a.Hq + h) * a.nq + min((kFastRows / BM) * iq + (wave >> 2), a.nq - 1)];
-    // k_scale is read through the constant address space: the loads stay scalar (s_load_dword) even though
-    // the loop contains assembly that clobbers memory, and they are tracked by lgkmcnt, not by the vmcnt
-    // the direct-to-LDS loads are tracked with
-    typedef __attribute__((address_space(4))) const float* const_f32_ptr;
-    const const_f32_ptr ksp = (const_f32_ptr)(uintptr_t)(a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk);
-    const int8_t* kg = a.k + (int64_t)b * a.ks_b + (int64_t)hk * a.ks_h;
-    const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
-
-    // ---- staging: direct-to-LDS loads, 16 bytes per lane, 1 KB per wave instruction.  LDS piece
-    //      p = 64 * instr + lane is chunk p % CPR of row p / CPR and receives the chunk (p % CPR) ^ swz(row)
-    //      of that row from global memory.  Wave w issues instructions w, w + 8, ... of a tile (a K tile of
-    //      head_dim 64 has only four, which waves 4-7 load a second time so that every wave has the same
-    //      number of loads in flight).  The swizzle of a wave's piece does not depend on which of its
-    //      instructions carries it (rows advance by a multiple of the swizzle period), so one per-lane
-    //      byte offset serves all of them and the instruction index only moves the uniform base.
-    static_assert(kFastWaves == 8 && F::V_INSTR % kFastWaves == 0, "load split");
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int k_idx = wave_u % F::K_INSTR;
-    unsigned k_goff, v_goff;
-    {
-        const int pk = 64 * k_idx + lane, rk = pk / F::KCPR;
-        k_goff = rk * (int)a.ks_n + 16 * ((pk % F::KCPR) ^ F::k_swz(rk));
-        const int pv = 64 * wave_u + lane, rv = pv / F::VCPR;
-        v_goff = rv * (int)a.vs_n * 2 + 16 * ((pv % F::VCPR) ^ F::v_swz(rv));
-    }
-    static_assert((64 * kFastWaves / F::KCPR) % (16 / F::KCPR * F::KCPR) == 0 && (64 * kFastWaves / F::VCPR) % 4 == 0, "swizzle period");
-    const int64_t k_instr_bytes = (int64_t)(64 * kFastWaves / F::KCPR) * a.ks_n;      // rows per round of the waves * row stride
-    const int64_t v_instr_bytes = (int64_t)(64 * kFastWaves / F::VCPR) * a.vs_n * 2;
-    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-    // The loads are written in assembly: the compiler would otherwise wait for every outstanding one
-    // before each LDS read that follows.  Completion is tracked by hand with s_waitcnt vmcnt.
-    auto dma16 = [](const unsigned char* base, unsigned voff, unsigned lds_addr) {
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");  // (m0 cannot be named as a clobber; nothing else in this kernel uses it)
-    };
-    // The last tile of a kv_len that is not a multiple of 64 (CAUSAL instance only): rows past the end
-    // re-read the last valid row (finite values under hidden scores), through per-lane offsets of their own.
-    const bool ragged = CAUSAL && (a.N % BN) != 0;
-    unsigned k_goff_last[F::NK], v_goff_last[F::NV];
-    if (CAUSAL) {
-        const int last = (a.N - 1) % BN;
-#pragma unroll
-        for (int e = 0; e < F::NK; e++) {
-            const int pk = 64 * k_idx + lane, rk = pk / F::KCPR + e * (64 * kFastWaves / F::KCPR);
-            k_goff_last[e] = min(rk, last) * (int)a.ks_n + 16 * ((pk % F::KCPR) ^ F::k_swz(rk));
-        }
-#pragma unroll
-        for (int e = 0; e < F::NV; e++) {
-            const int pv = 64 * wave_u + lane, rv = pv / F::VCPR + e * (64 * kFastWaves / F::VCPR);
-            v_goff_last[e] = min(rv, last) * (int)a.vs_n * 2 + 16 * ((pv % F::VCPR) ^ F::v_swz(rv));
-        }
-    }
-    // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions.
-    // kt / vt: index of the tile behind ktile / vtile
-    auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int kt, int vbuf, const unsigned char* vtile, int vt) {
-        constexpr int e = decltype(ec)::value;
-        if constexpr (e < F::NK) {
-            const bool cut = ragged && kt == a.nk - 1;
-            dma16(cut ? ktile : ktile + e * k_instr_bytes, cut ? k_goff_last[e] : k_goff,
-                  lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
-        } else {
-            constexpr int ev = e - F::NK;
-            const bool cut = ragged && vt == a.nk - 1;
-            dma16(cut ? vtile : vtile + ev * v_instr_bytes, cut ? v_goff_last[ev] : v_goff,
-                  lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
-        }
-    };
-    constexpr int NDMA = F::NK + F::NV;  // loads per wave per step
-
-    // ---- fragment read offsets (undoing the swizzle)
-    // K: lane (row l32, half) reads chunk half * D/32 + t of its row for k-step t
-    int kf_off[F::KSTEPS];
-#pragma unroll
-    for (int t = 0; t < F::KSTEPS; t++) kf_off[t] = l32 * F::K_RS + 16 * ((half * (D / 32) + t) ^ F::k_swz(l32));
-    // V, ds_read_b64_tr_b16: in each group of 16 lanes, lane 4s+a supplies keys row s, channels 4a..4a+3,
-    // and lane i receives channel i of the four rows.  Groups: (channels 0-15 | 16-31) x (half 0 | 1).
-    int vtr_off[F::DTILES];
-    {
-        const int s4 = (lane >> 2) & 3, a4 = lane & 3, g1 = (lane >> 4) & 1;
-#pragma unroll
-        for (int dt = 0; dt < F::DTILES; dt++)
-            vtr_off[dt] = (4 * half + s4) * F::V_RS + 16 * ((4 * dt + 2 * g1 + (a4 >> 1)) ^ F::v_swz(s4)) + 8 * (a4 & 1);
-    }
-
-    // The int32 accumulators start from the bit pattern of the float 1.5 * 2^23: since |dot| < 2^22,
-    // accumulator bits reinterpreted as fp32 ARE kBias + dot, so no int -> float conversion is needed.
-    v16i bias16;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        int b;  // materialised once through an opaque move, so the block stays in VGPRs for the whole kernel
-        asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "s"(kBiasBits));
-        bias16[i] = b;
-    }
-    auto qk_tile = [&](const unsigned char* kbase, int kt) {
-        v16i acc = bias16;
-#pragma unroll
-        for (int t = 0; t < F::KSTEPS; t++) {
-            const v4i kf = *reinterpret_cast<const v4i*>(kbase + kf_off[t] + 32 * kt * F::K_RS);
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[t], acc, 0, 0, 0);
-        }
-        return acc;
-    };
-
-    float m_i;         // reference point of the row's exponentials: set from the first tile below
-    float l_i = 0.0f;  // (the reference's initial l = 1 is multiplied by exp2(-inf) = 0 in its first step)
-    v16f o[F::DTILES];
-#pragma unroll
-    for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
-
-    // ---- the step pipeline -----------------------------------------------------------------
-    // The MFMA phase of a step issues QK_SLOTS + PV_SLOTS matrix instructions.  Each "slot" is one
-    // MFMA plus the few VALU / LDS instructions that run in its shadow, fenced so that the order
-    // written here is the order issued; LDS fragment reads are issued a few slots ahead of the
-    // MFMA that consumes them.
-    constexpr int QK_SLOTS = 2 * F::KSTEPS;
-    constexpr int PV_SLOTS = 4 * F::DTILES;
-    constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int DEFER = D == 64 ? 4 : 0;                   // exponential units moved into the MFMA phase
-    constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
-    constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
-    static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
-    static_assert(DEFER <= QK_SLOTS, "every P of a step exists when its row sums are checked, before the first P.V");
-
-    // Scores live in two register sets that swap roles every step (the loop body is instantiated
-    // for both parities), so the accumulators Q.K^T writes in one iteration are read in place by
-    // the exponentials of the next one.
-    v16i sbuf[2][2];  // [parity][32-key tile]: int32 accumulators whose bits are the float kBias + dot
-    float sc;         // q_scale * k_scale of the current step
-
-    auto as_f = [](int bits) { return __builtin_bit_cast(float, bits); };
-    auto head_unit = [&](auto pc, auto uc, int n0_next, bool masked, float& acc) {
-        constexpr int P = decltype(pc)::value, u = decltype(uc)::value;
-        constexpr int kt = u >> 2, i0 = 4 * (u & 3);
-        float x[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int bits = sbuf[P][kt][i0 + e];  // (scalar copy: bit_cast of a vector element lvalue reads element 0)
-            x[e] = as_f(bits);
-            if (CAUSAL && masked) {
-                const int i = i0 + e;
-                const int n = n0_next + 32 * kt + 8 * (i >> 2) + 4 * half + (i & 3);
-                x[e] = (n > lim) ? -INFINITY : x[e];
-                sbuf[P][kt][i] = __builtin_bit_cast(int, x[e]);
-            }
-        }
-        acc = fmaxf(fmaxf(acc, x[0]), x[1]);
-        acc = fmaxf(fmaxf(acc, x[2]), x[3]);
-        asm volatile("" ::"v"(acc));  // pin to this slot (otherwise sunk below the matrix instructions)
-    };
-    // The two lanes that share a row (l32 and l32 + 32) agree on the larger of their values.
-    auto row_pair_max = [](float x) {
-        const v2u sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, x), false, false);
-        const unsigned mine = sw[0], other = sw[1];  // (scalar copies: bit_cast of a vector element lvalue reads element 0)
-        return fmaxf(__builtin_bit_cast(float, mine), __builtin_bit_cast(float, other));
-    };
-
-    // ---- prologue: K0, K1, K2, V0, V1 in LDS; scores of step 0 in registers.  Tile indices past the
-    //      last step are clamped to it: such a tile is fetched again into a buffer nobody reads.
-    const int64_t k_tile_bytes = (int64_t)BN * a.ks_n, v_tile_bytes = (int64_t)BN * a.vs_n * 2;
-    const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg);
-    const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg);
-    int k_tile = 0, v_tile = 0;  // indices of the tiles behind k_fetch / v_fetch
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
-    if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
-    if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
-    sfor<F::NK>([&](auto ec) { dma_unit(ec, 2, k_fetch, k_tile, 2, v_fetch, v_tile); });
-    // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
-    if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
-    __syncthreads();
-    sbuf[0][0] = qk_tile(smem, 0);
-    sbuf[0][1] = qk_tile(smem, 1);
-    sc = qs * ksp[0];
-    if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
-    {   // the row maximum of the first tile is the reference point the row starts from
-        float raw_max = -INFINITY;
-        const bool masked0 = CAUSAL && (BN - 1 > wlim);
-        sfor<8>([&](auto uc) { head_unit(IC<0>{}, uc, 0, masked0, raw_max); });
-        m_i = (row_pair_max(raw_max) - kBias) * sc;
-    }
-
-    // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
-    // (Q.K^T of the next step, P.V of this one, with the row sums in the shadow of the matrix
-    // instructions); the two waves that share a SIMD run half a step
-    // apart (see the barrier before the loop), so one feeds the matrix core while the other
-    // occupies the VALU.  Two barriers per step.
-    auto body = [&](auto pc, int step) {
-        constexpr int P = decltype(pc)::value;  // == step & 1
-        // tile t of K (of V) lives in LDS buffer t % 4: this step reads K of step+1 and V of step, and
-        // fetches K of step+3 and V of step+2 into the buffers that K of step-1 and V of step-2 left
-        int kaddr[F::KSTEPS], vaddr[F::DTILES];
-#pragma unroll
-        for (int t = 0; t < F::KSTEPS; t++) {
-            kaddr[t] = kf_off[t] + ((step + 1) & 3) * F::K_BYTES;
-            asm volatile("" : "+v"(kaddr[t]));  // computed once per step, here in the VALU phase
-        }
-#pragma unroll
-        for (int dt = 0; dt < F::DTILES; dt++) {
-            vaddr[dt] = vtr_off[dt] + F::V_BASE + (step & 3) * F::V_BYTES;
-            asm volatile("" : "+v"(vaddr[dt]));
-        }
-        v4i kfr[QK_SLOTS];
-        vec16 vfr[PV_SLOTS];
-        auto read_k = [&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            kfr[i] = *reinterpret_cast<const v4i*>(smem + kaddr[i / 2] + 32 * (i % 2) * F::K_RS);
-        };
-        auto read_v = [&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const unsigned char* p0 = smem + vaddr[j % F::DTILES] + 16 * (j / F::DTILES) * F::V_RS;
-            vfr[j] = tr_pair<VT>(p0, p0 + 8 * F::V_RS);
-        };
-        const int n0 = step * BN;
-        const bool live = step < nsteps;  // false only for the padding step after an odd number of steps
-
-        // ===== VALU phase: exponentials of this step (scores in sbuf[P]) =====
-        // No row maximum is taken: the exponentials use the reference point m_i the row already has, which
-        // any value not far below the true maximum serves equally well (the result is O / l either way).
-        // Should it make a P too large, the row sums show it before the first P.V instruction, and the step
-        // is redone against its true maximum: see redo_if_large below.
-        float neg_m;
-        const bool folded = kBias * sc < kBiasFoldLimit;
-        if (folded) {
-            neg_m = __builtin_fmaf(-kBias, sc, -m_i);
-        } else {
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int bits = sbuf[P][kt][i];
-                    sbuf[P][kt][i] = __builtin_bit_cast(int, as_f(bits) - kBias);
-                }
-            neg_m = -m_i;
-        }
-        if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
-        // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
-        // instruction.
-        sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
-        vec16 pf[4];
-        float lsum = 0.0f;
-        const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
-        auto exp_unit = [&](auto uc) {  // two scores -> two 16-bit P values
-            constexpr int u = decltype(uc)::value;
-            constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
-            const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
-            pf[tp][2 * w] = (VT)p0;
-            pf[tp][2 * w + 1] = (VT)p1;
-        };
-        // The last DEFER of the 16 units wait for the MFMA phase (head_dim 64: that phase has half the
-        // matrix instructions, so it takes a share of the exponentials to keep the two phases even).
-        sfor<16 - DEFER>(exp_unit);
-        // A lane's 32 P of a step sum to less than kSumLimit, or the step is redone: so no P overflows the
-        // 16-bit type (nor does a sum or a product with V come near the fp32 range), and a row whose scores
-        // rise keeps its reference point within log2(kSumLimit) of its maximum.  Wave-wide decision; rare
-        // after the first steps of a row (the maximum of a row rises ever more slowly).
-        auto redo_if_large = [&]() {
-            if (__builtin_amdgcn_ballot_w64(!(lsum < kSumLimit)) != 0) {  // also taken for inf and NaN
-                float raw = -INFINITY;
-#pragma unroll
-                for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int bits = sbuf[P][kt][i];
-                        raw = fmaxf(raw, as_f(bits));
-                    }
-                const float rmax = (row_pair_max(raw) - (folded ? kBias : 0.0f)) * sc_e;
-                const float m_new = fmaxf(m_i, rmax);
-                const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-                l_i *= alpha;
-                m_i = m_new;
-#pragma unroll
-                for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
-                neg_m = folded ? __builtin_fmaf(-kBias, sc_e, -m_i) : -m_i;
-                lsum = 0.0f;
-                sfor<16>([&](auto uc) {
-                    constexpr int u = decltype(uc)::value;
-                    exp_unit(uc);
-                    lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
-                });
-            }
-        };
-        sc = qs * ksp[min(step + 1, nsteps - 1)];
-        if (CAUSAL) sc = fmaxf(sc, 1.17549435e-38f);
-        __builtin_amdgcn_sched_barrier(0);
-        // The first K fragments of the coming MFMA phase are requested before the barrier (their tile
-        // landed a step ago), so the phase does not open with an LDS round trip.
-        sfor<KDIST>(read_k);
-        __builtin_amdgcn_sched_barrier(0);
-        // The loads issued in the previous VALU phase have landed (all but the NDMA just issued): the
-        // tiles they belong to are first read two barriers from here.
-        __builtin_amdgcn_s_waitcnt(0x0F70 | NDMA);
-        __builtin_amdgcn_s_barrier();        // phase switch: this wave takes the matrix core
-        __builtin_amdgcn_sched_barrier(0);
-
-        // ===== MFMA phase =====
-        __builtin_amdgcn_s_setprio(1);
-        const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > wlim);
-        sfor<NSLOTS>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            if constexpr (i < QK_SLOTS) {
-                constexpr int kt = i % 2, t = i / 2;  // alternate the two accumulation chains
-                if constexpr (t == 0) {
-                    sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], bias16, 0, 0, 0);
-                } else {
-                    sbuf[1 - P][kt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfr[i], qf[t], sbuf[1 - P][kt], 0, 0, 0);
-                }
-                if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
-                if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
-                // row sums of P ride in the shadow of the Q.K^T instructions
-                sfor<16 - DEFER>([&](auto rc) {
-                    constexpr int u = decltype(rc)::value;
-                    if constexpr (u * QK_SLOTS / (16 - DEFER) == i) {
-                        lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
-                        asm volatile("" ::"v"(lsum));
-                    }
-                });
-            } else {
-                constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
-                if constexpr (j == 0) {
-                    redo_if_large();
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                o[dt] = PVT::mfma(vfr[j], pf[tp], o[dt]);
-                if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
-                // hidden keys of the next step's scores (Q.K^T finished above) are set to -inf under the
-                // P.V instructions
-                if constexpr (CAUSAL) {
-                    sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
-                        constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
-                        if constexpr (u < 8) {
-                            float unused = 0.0f;
-                            if (masked_n) head_unit(IC<1 - P>{}, IC<u>{}, n0 + BN, true, unused);
-                        }
-                    });
-                }
-            }
-            if constexpr (i < DEFER) {  // a deferred exponential unit and its row-sum term
-                constexpr int u = 16 - DEFER + i;
-                static_assert(DEFER == 0 || QK_SLOTS + (u >> 2) * F::DTILES > i, "P is ready before the P.V slot that multiplies with it");
-                exp_unit(IC<u>{});
-                lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
-                asm volatile("" ::"v"(lsum));
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        l_i += lsum;
-        if (step + 4 < nsteps) { k_fetch += k_tile_bytes; k_tile++; }  // next iteration fetches K of step+4, V of step+3
-        if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
-        __builtin_amdgcn_s_setprio(0);
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
-        __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    if (wave >= kFastWaves / 2) __syncthreads();  // second half of the waves runs one phase behind
-    // The loop always runs an even number of steps (no exit between the two parities: the accumulators
-    // then stay in one set of registers); after an odd nsteps the extra step multiplies V by P = 0.
-    for (int step = 0; step < nsteps; step += 2) {
-        body(IC<0>{}, step);
-        body(IC<1>{}, step + 1);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // every direct-to-LDS load of this wave has landed
-    if (wave < kFastWaves / 2) __syncthreads();
-    __syncthreads();  // nobody reads or fills a K/V tile any more: the LDS is free for the output
-    // ---- epilogue: O = O^T / l, lse = log2(l) + m
-    const float l_o = __shfl_xor(l_i, 32);
-    const float l_tot = half ? (l_o + l_i) : (l_i + l_o);
-    const float inv = 1.0f / l_tot;
-    const int64_t obase_wave = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)(m0 + 32 * wave) * a.os_n;
-    if (a.out_dt != SAGE_F32) {
-        // 16-bit outputs: a lane holds its row in 8-byte pieces, which stored directly would scatter 32
-        // partial lines per instruction.  Each wave transposes its 32 rows through its own slice of LDS
-        // and writes whole rows, 16 bytes per lane.
-        constexpr int ORS = 2 * D + 16;  // bytes per staged row
-        static_assert(kFastWaves * 32 * ORS <= F::TOTAL, "output staging fits in the tile buffers");
-        unsigned char* mine = smem + wave * 32 * ORS;
-#pragma unroll
-        for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                float r[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) r[i] = o[dt][4 * g + i] * inv;
-                s16x4 w;
-                if (a.out_dt == SAGE_BF16) {
-                    typedef __bf16 b4 __attribute__((ext_vector_type(4)));
-                    w = __builtin_bit_cast(s16x4, b4{(__bf16)r[0], (__bf16)r[1], (__bf16)r[2], (__bf16)r[3]});
-                } else {
-                    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-                    w = __builtin_bit_cast(s16x4, h4{(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]});
-                }
-                *reinterpret_cast<s16x4*>(mine + l32 * ORS + 2 * (32 * dt + 8 * g + 4 * half)) = w;
-            }
-        asm volatile("" ::: "memory");  // the reads below see other lanes' writes (same wave: LDS keeps program order)
-        constexpr int LPR = 2 * D / 16, RPI = 64 / LPR;  // lanes per row, rows per wave instruction
-        unsigned char* outp = reinterpret_cast<unsigned char*>(a.out) + 2 * obase_wave + 16 * (lane % LPR);
-#pragma unroll
-        for (int e = 0; e < 32 / RPI; e++) {
-            const int r = RPI * e + lane / LPR;
-            const v4i piece = *reinterpret_cast<const v4i*>(mine + r * ORS + 16 * (lane % LPR));
-            if (m0 + 32 * wave + r < a.M) *reinterpret_cast<v4i*>(outp + 2 * (int64_t)r * a.os_n) = piece;
-        }
-    } else if (row_ok) {
-        float* outp = static_cast<float*>(a.out) + obase_wave + (int64_t)l32 * a.os_n;
-#pragma unroll
-        for (int dt = 0; dt < F::DTILES; dt++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d = 32 * dt + 8 * g + 4 * half;
-                *reinterpret_cast<v4f*>(outp + d) = v4f{o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv, o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv};
-            }
-    }
-    if (row_ok) {
-        if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = __builtin_log2f(l_tot) + m_i;
-    }
-}
 
 template <int D, typename VT>
 int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
@@ -570,8 +40,8 @@ int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
     const int nq2 = (a.M + kFastRows - 1) / kFastRows;
     b.total_wg = (int)((int64_t)a.total_wg / a.nq * nq2);
     dim3 grid((unsigned)b.total_wg), block(kFastThreads);
-    if (causal) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true>), grid, block, 0, stream, b, nq2);
-    else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false>), grid, block, 0, stream, b, nq2);
+    if (causal) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1>), grid, block, 0, stream, b, nq2);
+    else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false, 1>), grid, block, 0, stream, b, nq2);
     return check_launch("sage_attn_fwd_fast_kernel");
 }
 

@@ -1,0 +1,81 @@
+"""Dense attention forward on MI355X behind the signature of FlagAttention's ``flash_attention``
+(src/flag_attn/flash.py:275-306): ``attention(q, k, v, causal=False, sm_scale=None, ...)`` on
+(batch, heads, sequence, head_dim) tensors of any strides with a unit innermost stride.
+
+Built here: the forward pass for fp16 / bf16, head_dim 64 or 128, grouped K/V heads, the causal flag
+for any qo_len / kv_len (bottom-right aligned, flash.py:53-54), ``sm_scale`` and the natural-log
+log normalizer (flash.py:503-506).  Not built: dropout, the total attention, head_dim 16 / 32 and the
+backward pass; a call that asks for one of them raises instead of computing something else.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from .sage_attention._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, tensor_desc
+
+__all__ = ["attention"]
+
+
+def _rows16(t: torch.Tensor) -> torch.Tensor:
+    # the kernel loads 16 bytes per lane: rows start on 16-byte boundaries and run along the last axis
+    return t if rows_aligned(t) else t.contiguous()
+
+
+def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
+              return_log_normalizer=False, return_total_attention=False, return_seed_offset=False):
+    """O = softmax(sm_scale * Q K^T [causal]) V, and optionally logsumexp(sm_scale * Q K^T) per query.
+
+    Returns ``o`` alone, or the reference's 5-tuple ``(o, log_normalizer, None, None, None)`` when an
+    extra output is asked for (flash.py:170-180).
+    """
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be (batch, heads, sequence, head_dim) tensors")
+    Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    Hk, Hv = k.shape[1], v.shape[1]
+    assert Hk == Hv, "num of heads in k and v should be equal"
+    assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+    if k.shape[0] != B or v.shape[0] != B or v.shape[2] != N:
+        raise ValueError("batch and sequence sizes of q, k, v do not match")
+    if dropout_p != 0.0 or return_seed_offset:
+        raise NotImplementedError("flagattention_amd.flash.attention: dropout is not built")
+    if return_total_attention:
+        raise NotImplementedError("flagattention_amd.flash.attention: the total attention is not built")
+    if D not in (64, 128):
+        raise NotImplementedError(f"flagattention_amd.flash.attention: head_dim {D} is not built (64 or 128)")
+    if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("q, k, v must share one of torch.float16 / torch.bfloat16")
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        raise NotImplementedError("flagattention_amd.flash.attention: forward only (no backward pass is built); "
+                                  "call it under torch.no_grad() or on tensors that do not require grad")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        require_gpu(t, name)
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    if M == 0 or N == 0 or B == 0:
+        raise ValueError("empty q or k")
+
+    q, k, v = _rows16(q), _rows16(k), _rows16(v)
+    o = torch.empty_like(q)  # (the reference allocates the same way, flash.py:84-90)
+    if not rows_aligned(o):
+        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    L = torch.empty((B, H, M), dtype=torch.float32, device=q.device) if return_log_normalizer else None
+
+    p = _lib.FlashParams()
+    p.q, p.k, p.v, p.out = (tensor_desc(t, True) for t in (q, k, v, o))
+    p.log_normalizer = L.data_ptr() if L is not None else None
+    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = B, H, Hk, M, N, D
+    p.dtype = p.out_dtype = DTYPE_CODE[q.dtype]
+    p.causal = 1 if causal else 0
+    p.sm_scale = float(sm_scale)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        _lib.check(lib.sage_flash_attn_fwd(p, current_stream_ptr(q.device)), "sage_flash_attn_fwd")
+    if return_log_normalizer:
+        return o, L, None, None, None
+    return o

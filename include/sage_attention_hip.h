@@ -1,5 +1,6 @@
 /*
- * C ABI of libsage_attention_hip.so: FlagAttention's SageAttention path on MI355X (gfx950).
+ * C ABI of libsage_attention_hip.so: FlagAttention's SageAttention path on MI355X (gfx950), and the
+ * dense 16-bit attention forward that shares its kernel.
  *
  * Plain pointers, sizes and strides only; no framework types.  All pointers are device
  * pointers on the current HIP device unless stated otherwise; strides are in ELEMENTS and the
@@ -104,12 +105,36 @@ int64_t sage_k_mean_workspace_bytes(int64_t batch, int64_t heads_kv, int64_t kv_
 int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out_dtype, int64_t batch,
                 int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* workspace, void* stream);
 
+/*
+ * Dense attention forward on 16-bit Q, K, V: replaces the forward launch of FlagAttention's
+ * flash_attention (src/flag_attn/flash.py:37-180 host, :346-510 kernel) for the calls that need no
+ * dropout, no total attention and no gradient:  O = softmax(sm_scale * Q K^T [+ causal]) V.
+ *
+ *   q, k, v      dtype (SAGE_F16 / SAGE_BF16), own strides (any of the two layouts, GQA by heads_kv)
+ *   out          out_dtype (SAGE_F16 / SAGE_BF16 / SAGE_F32), own strides
+ *   log_normalizer  optional [B, Hq, M] fp32 contiguous: natural-log log-sum-exp of the scaled scores
+ *                (flash.py:503-506); NULL = none
+ *   causal       non-zero: key n is visible to query m iff n <= m + (N - M) (flash.py:53-54, P_SEQ);
+ *                a query that sees no key (M > N) yields a zero row and a log normalizer of -inf
+ *   sm_scale     factor on Q K^T (the host passes 1/sqrt(head_dim) by default, flash.py:57-58)
+ * head_dim must be 64 or 128 (the reference also takes 16 and 32); heads_q a multiple of heads_kv.
+ */
+typedef struct sage_flash_params {
+    sage_tensor q, k, v, out;
+    float* log_normalizer;
+    int64_t batch, heads_q, heads_kv, qo_len, kv_len, head_dim;
+    int32_t dtype, out_dtype, causal;
+    float sm_scale;
+} sage_flash_params;
+
+int sage_flash_attn_fwd(const sage_flash_params* p, void* stream);
+
 /* Message describing the last non-zero status returned on this thread ("" if none). */
 const char* sage_hip_last_error(void);
 
 /* ABI version of this header; bumped when a struct layout changes. */
 int sage_hip_abi_version(void);
-#define SAGE_HIP_ABI_VERSION 1
+#define SAGE_HIP_ABI_VERSION 2
 
 #ifdef __cplusplus
 }

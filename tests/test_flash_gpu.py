@@ -1,0 +1,140 @@
+"""GPU parity of the dense attention forward (flag_attn.flash_attention) against the CPU oracle.
+
+Acceptance rule of the reference's own test (tests/flag_attn/test_flash_attention.py:116-124):
+the kernel's largest deviation from the fp32 closed form may be at most twice that of the same
+closed form evaluated in the inputs' 16-bit dtype, plus 1e-5.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import flash_oracle as FO
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(seed, B, Hq, Hk, M, N, D, dtype, order="BHTD", std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    if order == "BHTD":
+        q = torch.randn(B, Hq, M, D, generator=g).mul_(std).to(dtype)
+        k = torch.randn(B, Hk, N, D, generator=g).mul_(std).to(dtype)
+        v = torch.randn(B, Hk, N, D, generator=g).mul_(std).to(dtype)
+    else:  # stored (B, T, H, D), seen as (B, H, T, D)
+        q = torch.randn(B, M, Hq, D, generator=g).mul_(std).to(dtype).transpose(1, 2)
+        k = torch.randn(B, N, Hk, D, generator=g).mul_(std).to(dtype).transpose(1, 2)
+        v = torch.randn(B, N, Hk, D, generator=g).mul_(std).to(dtype).transpose(1, 2)
+    return q, k, v
+
+
+def _check(q, k, v, causal, dev, sm_scale=None):
+    import flag_attn
+
+    o, L, *rest = flag_attn.flash_attention(q.to(dev), k.to(dev), v.to(dev), causal, sm_scale=sm_scale,
+                                            return_log_normalizer=True)
+    torch.cuda.synchronize()
+    assert rest == [None, None, None] and o.dtype == q.dtype and o.shape == q.shape
+    o_ref, L_ref = FO.attention(q, k, v, causal, sm_scale=sm_scale, return_log_normalizer=True, upcast=True)
+    o_16 = FO.attention(q, k, v, causal, sm_scale=sm_scale, upcast=False)
+    yard = FO.max_diff(o_16, o_ref)
+    got = FO.max_diff(o.cpu(), o_ref)
+    assert got <= 2 * yard + 1e-5, f"max diff {got} against a 16-bit yardstick of {yard}"
+    inf = torch.isinf(L_ref)
+    assert torch.equal(torch.isinf(L.cpu()), inf)
+    # the reference's rule for the log normalizer is relative to a 16-bit evaluation as well (:290-291);
+    # an fp32-accumulating kernel is held to a fixed bound instead
+    torch.testing.assert_close(L.cpu()[~inf], L_ref[~inf], atol=2e-3, rtol=2e-4)
+    return o
+
+
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", [
+    (2, 4, 4, 512, 612, 128),
+    (2, 4, 4, 1024, 1034, 64),
+    (1, 4, 4, 1001, 1001, 64),
+    (1, 4, 4, 1001, 1024, 64),
+    (2, 4, 4, 1024, 1000, 128),   # more queries than keys: under the causal flag the first 24 see none
+    (2, 4, 2, 512, 612, 128),     # grouped K/V heads
+    (2, 4, 1, 1024, 1034, 64),
+    (1, 4, 1, 1001, 1024, 64),
+    (2, 4, 2, 1024, 1000, 128),
+])
+def test_forward_against_reference_rule(B, Hq, Hk, M, N, D, causal, dtype, order, gpu_device):
+    q, k, v = _inputs(1, B, Hq, Hk, M, N, D, dtype, order)
+    _check(q, k, v, causal, gpu_device)
+
+
+@pytest.mark.parametrize("std", [2.0, 4.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_forward_input_scales(std, causal, gpu_device):
+    """The reference sweeps the standard deviation of the inputs up to 4 (:80): scores reach +-500."""
+    q, k, v = _inputs(2, 2, 4, 2, 640, 700, 128, torch.bfloat16, std=std)
+    _check(q, k, v, causal, gpu_device)
+
+
+@pytest.mark.parametrize("M,N", [(1, 1), (1, 612), (2, 1000), (4, 2058), (300, 64), (64, 63), (257, 130)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_forward_small_and_ragged_shapes(M, N, causal, gpu_device):
+    q, k, v = _inputs(3, 2, 4, 2, M, N, 64, torch.float16)
+    _check(q, k, v, causal, gpu_device)
+    q, k, v = _inputs(4, 1, 2, 2, M, N, 128, torch.bfloat16)
+    _check(q, k, v, causal, gpu_device)
+
+
+def test_sm_scale_and_known_answers(gpu_device):
+    import flag_attn
+
+    q, k, v = _inputs(5, 1, 2, 2, 256, 320, 128, torch.float16)
+    _check(q, k, v, False, gpu_device, sm_scale=0.05)
+    _check(q, k, v, True, gpu_device, sm_scale=0.3)
+    # q = 0: uniform softmax, o = mean of V, log normalizer = log(N); under the causal flag the mean of
+    # the visible prefix and log(its length)
+    z = torch.zeros_like(q)
+    o, L, *_ = flag_attn.flash_attention(z.to(gpu_device), k.to(gpu_device), v.to(gpu_device), False, return_log_normalizer=True)
+    torch.testing.assert_close(o.float().cpu(), v.float().mean(2, keepdim=True).expand(-1, -1, 256, -1), atol=2e-3, rtol=2e-3)
+    torch.testing.assert_close(L.cpu(), torch.full((1, 2, 256), math.log(320.0)), atol=1e-3, rtol=1e-4)
+    o, L, *_ = flag_attn.flash_attention(z.to(gpu_device), k.to(gpu_device), v.to(gpu_device), True, return_log_normalizer=True)
+    visible = torch.arange(256) + 65.0  # row m sees keys 0 .. m + 64
+    torch.testing.assert_close(L.cpu(), visible.log().expand(1, 2, -1), atol=1e-3, rtol=1e-4)
+    prefix_mean = v.float().cumsum(2)[:, :, 64:] / visible.view(1, 1, -1, 1)
+    torch.testing.assert_close(o.float().cpu(), prefix_mean, atol=3e-3, rtol=3e-3)
+    # single return value when no extra output is asked for
+    o2 = flag_attn.flash_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))
+    assert isinstance(o2, torch.Tensor)
+
+
+def test_unbuilt_features_raise(gpu_device):
+    import flag_attn
+
+    q, k, v = (t.to(gpu_device) for t in _inputs(6, 1, 2, 2, 64, 64, 64, torch.float16))
+    with pytest.raises(NotImplementedError):
+        flag_attn.flash_attention(q, k, v, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        flag_attn.flash_attention(q, k, v, return_total_attention=True)
+    with pytest.raises(NotImplementedError):
+        flag_attn.flash_attention(q[..., :32], k[..., :32], v[..., :32])
+    with pytest.raises(NotImplementedError):
+        flag_attn.flash_attention(q.requires_grad_(), k, v)
+    with pytest.raises(AssertionError):
+        flag_attn.flash_attention(q, k[:, :1], v)
+
+
+def test_full_size_llama_shape(gpu_device):
+    """B4 H32 N4096 D128 bf16 (the shape the SageAttention benchmark is quoted on): two heads against the
+    oracle; every head against the property that rows of O are convex combinations of rows of V."""
+    import flag_attn
+
+    g = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(4, 32, 4096, 128, generator=g).to(torch.bfloat16) for _ in range(3))
+    o = flag_attn.flash_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), False)
+    torch.cuda.synchronize()
+    for (b, h) in [(0, 0), (3, 31)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = FO.attention(q[sl], k[sl], v[sl], False, upcast=True)
+        yard = FO.max_diff(FO.attention(q[sl], k[sl], v[sl], False, upcast=False), ref)
+        assert FO.max_diff(o[sl].cpu(), ref) <= 2 * yard + 1e-5
+    vmax = v.to(gpu_device).float().amax(2, keepdim=True)
+    vmin = v.to(gpu_device).float().amin(2, keepdim=True)
+    assert bool(torch.isfinite(o).all()) and bool((o.float() <= vmax + 1e-2).all()) and bool((o.float() >= vmin - 1e-2).all())

@@ -201,3 +201,66 @@ def test_config1_cpu_plumbing():
     base = O.sdpa_cpu_baseline(q, k, v, output_dtype=torch.float16)
     cos, rel, _ = O.accuracy_metrics(out, base)
     assert cos >= 0.99 and rel <= 0.05  # the reference benchmark's own gate
+
+
+# ---- dense flash_attention oracle ------------------------------------------------------------
+
+def _brute_force_attention(q, k, v, causal, sm_scale):
+    """Loop over (query, key) pairs in float64: softmax over the visible keys, zero row if none."""
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    o = torch.zeros(B, H, M, D, dtype=torch.float64)
+    lse = torch.full((B, H, M), float("-inf"), dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            hk = h // (H // Hk)
+            for m in range(M):
+                keys = [n for n in range(N) if (not causal) or n <= m + (N - M)]
+                if not keys:
+                    continue
+                s = [sm_scale * float(q[b, h, m].double() @ k[b, hk, n].double()) for n in keys]
+                top = max(s)
+                w = [math.exp(x - top) for x in s]
+                tot = sum(w)
+                lse[b, h, m] = top + math.log(tot)
+                for x, n in zip(w, keys):
+                    o[b, h, m] += (x / tot) * v[b, hk, n].double()
+    return o, lse
+
+
+def test_flash_oracle_reduces_to_sdpa():
+    from oracle import flash_oracle as FO
+
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, 4, 96, 64, generator=g) for _ in range(3))
+    for causal in (False, True):
+        o, lse = FO.attention(q, k, v, causal=causal, sm_scale=0.2, return_log_normalizer=True)
+        ref = F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=0.2)
+        torch.testing.assert_close(o, ref, atol=2e-6, rtol=1e-5)
+        s = (q @ k.transpose(2, 3)).double() * 0.2
+        if causal:
+            s = s.masked_fill(~torch.ones(96, 96, dtype=torch.bool).tril(), float("-inf"))
+        torch.testing.assert_close(lse.double(), s.exp().sum(-1).log(), atol=1e-5, rtol=1e-6)
+    # default scale 1/sqrt(D); grouped K/V heads repeat each K/V head over consecutive query heads
+    o = FO.attention(q, k[:, :2], v[:, :2])
+    ref = F.scaled_dot_product_attention(q, k[:, :2].repeat_interleave(2, 1), v[:, :2].repeat_interleave(2, 1))
+    torch.testing.assert_close(o, ref, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("m,n", [(5, 9), (9, 5), (7, 7), (1, 6), (6, 1)])
+def test_flash_oracle_causal_alignment_brute_force(m, n):
+    """Bottom-right alignment for M != N, zero rows and -inf log normalizer where a query sees no key
+    (M > N): a top-left aligned mask, a dropped N - M or a NaN row would all fail here."""
+    from oracle import flash_oracle as FO
+
+    g = torch.Generator().manual_seed(10 * m + n)
+    q = torch.randn(1, 2, m, 8, generator=g)
+    k, v = torch.randn(1, 1, n, 8, generator=g), torch.randn(1, 1, n, 8, generator=g)
+    o, lse = FO.attention(q, k, v, causal=True, sm_scale=0.7, return_log_normalizer=True)
+    bo, blse = _brute_force_attention(q, k, v, True, 0.7)
+    torch.testing.assert_close(o.double(), bo, atol=1e-5, rtol=1e-5)
+    assert torch.equal(torch.isinf(lse), torch.isinf(blse))
+    fin = torch.isfinite(blse)
+    torch.testing.assert_close(lse.double()[fin], blse[fin], atol=1e-5, rtol=1e-6)
+    if m > n:
+        assert float(o[:, :, : m - n].abs().max()) == 0.0
