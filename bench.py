@@ -2,6 +2,7 @@
 """Benchmark of the SageAttention hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5] [--no-cpu]
+    python bench.py --op flash_attention [...]      (the sibling dense 16-bit forward, same shapes)
 
 One "step" is one pass of the hot path over one batch resident in HBM:
 K mean (fixed order) -> fused smoothing + per-block INT8 quantization of Q and K -> INT8-QK
@@ -102,12 +103,86 @@ def cpu_baseline(name, q, k, v, budget_s=12.0):
     }
 
 
+def main_flash(args):
+    """--op flash_attention: one step = one dense 16-bit attention forward (flag_attn.flash_attention) on the
+    workload's Q, K, V resident in HBM; 4*B*H*M*N*D flops (causal: visible pairs only) against the dense
+    16-bit MFMA peak."""
+    import flag_attn
+    from oracle import flash_oracle as FO
+
+    dev = torch.device("cuda:0")
+    name = args.workload
+    b, h, n, d, dtype, layout, causal, desc = WORKLOADS[name]
+    q0, k0, v0 = make_inputs(name, dev)
+    # the dense operator takes (batch, heads, sequence, head_dim) views of any strides
+    q, k, v = ((t.transpose(1, 2) if layout == "NHD" else t) for t in (q0, k0, v0))
+    qd, kd, vd = ((t.to(dev).transpose(1, 2) if layout == "NHD" else t.to(dev)) for t in (q0, k0, v0))
+
+    def step():
+        return flag_attn.flash_attention(qd, kd, vd, causal)
+
+    o = step()
+    torch.cuda.synchronize()
+    parity = None
+    if n <= 8192:  # one (batch, head) against the CPU oracle, under the reference's acceptance rule
+        sl = (slice(0, 1), slice(0, 1))
+        ref = FO.attention(q[sl], k[sl], v[sl], causal, upcast=True)
+        yard = FO.max_diff(FO.attention(q[sl], k[sl], v[sl], causal, upcast=False), ref)
+        got = FO.max_diff(o[sl].cpu(), ref)
+        parity = {"max_diff": got, "max_diff_of_16bit_closed_form": yard, "within_reference_rule": got <= 2 * yard + 1e-5,
+                  "checked_on": "batch 0, head 0 vs the CPU oracle"}
+    t_ramp = time.perf_counter()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ramp_steps = 0
+    while time.perf_counter() - t_ramp < 0.15:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        ramp_steps += 10
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e in events:
+        e[0].record()
+        step()
+        e[1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    launch_ms = [e[0].elapsed_time(e[1]) for e in events]
+    avg = sum(launch_ms) / len(launch_ms)
+    ms_per_step = wall / args.steps * 1e3
+    ops = algorithmic_ops(name)
+    numel = b * h * n * d
+    result = {
+        "metric": "TFLOP/s of the dense 16-bit attention forward (4*B*H*M*N*D flops per call; causal: visible pairs only)",
+        "value": round(ops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "clock_ramp_steps": ramp_steps,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if dtype == torch.bfloat16 else "f16", "data": "synthetic (seed 42, generated on CPU, copied to HBM before timing)",
+        "config": {"workload": "flash_attention_" + desc.split("_smoothk")[0], "batch": b, "heads": h, "seq_len": n, "head_dim": d,
+                   "layout": layout, "causal": causal},
+        "parity": parity,
+        "roofline": {"kernel": "sage_attn_fwd_fast_kernel (16-bit Q, K instance)", "bound": "mfma",
+                     "achieved": round(ops / (avg * 1e-3) / 1e12, 2), "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": 4 * numel * 2, "algorithmic_ops_per_launch": ops,
+                     "avg_launch_ms": round(avg, 4)},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(name, q0, k0, v0)
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--op", default="sage_attention", choices=["sage_attention", "flash_attention"],
+                    help="sage_attention (default): K mean + quantization + INT8-QK forward; flash_attention: the dense 16-bit forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed region, run 3 device-to-device tensor copies of this many MiB "
@@ -120,6 +195,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+
+    if args.op == "flash_attention":
+        return main_flash(args)
 
     from flag_attn import sage_attention as sa
     from oracle import sage_oracle as O
