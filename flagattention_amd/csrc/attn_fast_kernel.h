@@ -81,20 +81,30 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     using vec16 = typename PVT::vec;
     __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
 
-    const int tid = threadIdx.x;
+
+    // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
+    // Under the causal flag a workgroup takes two q-blocks of its head, one after the other: block
+    // nq2 - 1 - j (long rows) and block j (short rows), so that every workgroup of the launch runs about
+    // the same number of steps (one q-block alone runs between 1/nq2 and all of them).
+    int wg = blockIdx.x;
+    if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
+    const bool paired = CAUSAL && a.causal;
+    const int per_head = paired ? (nq2 + 1) / 2 : nq2;  // workgroups per (batch, head)
+    const int jq = wg % per_head;
+    const int h = (wg / per_head) % a.Hq;
+    const int b = wg / (per_head * a.Hq);
+    const int hk = h / a.groups;
+  for (int pass = 0; pass < 2; pass++) {
+    if (pass == 1 && (!paired || nq2 - 1 - jq == jq)) break;  // one q-block only, or the middle one of an odd count
+    // Everything a pass needs is derived again from the thread index, made opaque here: values the compiler
+    // would otherwise keep across the two passes cost registers the step loop cannot spare.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     const int wave = tid >> 6;
     const int lane = tid & 63;
     const int l32 = lane & 31;
     const int half = lane >> 5;
-
-    // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
-    int wg = blockIdx.x;
-    if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
-    int iq = wg % nq2;
-    if (CAUSAL && a.causal) iq = nq2 - 1 - iq;  // longest rows first
-    const int h = (wg / nq2) % a.Hq;
-    const int b = wg / (nq2 * a.Hq);
-    const int hk = h / a.groups;
+    const int iq = paired && pass == 0 ? nq2 - 1 - jq : jq;
     const int m0 = iq * kFastRows;
     const int my_m = m0 + 32 * wave + l32;
     const bool row_ok = my_m < a.M;
@@ -558,6 +568,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     if (row_ok) {
         if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = (__builtin_log2f(l_tot) + m_i) * a.lse_mul;
     }
+    __syncthreads();  // the output staging in LDS has been read: the next q-block may fill the tile buffers
+  }
 }
 
 }  // namespace

@@ -14,9 +14,12 @@ namespace {
 template <int D, typename VT>
 int launch_dense(const AttnArgs& a, bool hides_keys, hipStream_t stream) {
     const int nq2 = (a.M + kFastRows - 1) / kFastRows;
-    dim3 grid((unsigned)a.total_wg), block(kFastThreads);
-    if (hides_keys) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 2>), grid, block, 0, stream, a, nq2);
-    else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false, 2>), grid, block, 0, stream, a, nq2);
+    AttnArgs b = a;
+    const int per_head = a.causal ? (nq2 + 1) / 2 : nq2;  // under the causal flag a workgroup takes two q-blocks
+    b.total_wg = (int)((int64_t)a.total_wg / nq2 * per_head);
+    dim3 grid((unsigned)b.total_wg), block(kFastThreads);
+    if (hides_keys) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 2>), grid, block, 0, stream, b, nq2);
+    else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false, 2>), grid, block, 0, stream, b, nq2);
     return check_launch("sage_attn_fwd_fast_kernel (16-bit Q, K)");
 }
 
