@@ -138,3 +138,41 @@ def test_full_size_llama_shape(gpu_device):
     vmax = v.to(gpu_device).float().amax(2, keepdim=True)
     vmin = v.to(gpu_device).float().amin(2, keepdim=True)
     assert bool(torch.isfinite(o).all()) and bool((o.float() <= vmax + 1e-2).all()) and bool((o.float() >= vmin - 1e-2).all())
+
+
+def _sweep_cases():
+    import random
+
+    rnd = random.Random(20260101)
+    cases = []
+    for i in range(40):
+        hk = rnd.choice([1, 2, 3])
+        cases.append(dict(seed=100 + i, B=rnd.choice([1, 2]), Hk=hk, Hq=hk * rnd.choice([1, 2, 4]),
+                          M=rnd.choice([1, 3, 31, 64, 65, 127, 255, 256, 257, 300, 513, 700]),
+                          N=rnd.choice([1, 2, 63, 64, 65, 100, 128, 191, 320, 449, 512, 777]),
+                          D=rnd.choice([64, 128]), dtype=rnd.choice([torch.float16, torch.bfloat16]),
+                          causal=rnd.random() < 0.5, order=rnd.choice(["BHTD", "BTHD"]),
+                          std=rnd.choice([0.5, 1.0, 3.0])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: "b{B}_hq{Hq}_hk{Hk}_m{M}_n{N}_d{D}_{order}_c{causal}_s{std}".format(**c))
+def test_seeded_shape_sweep(case, gpu_device):
+    q, k, v = _inputs(case["seed"], case["B"], case["Hq"], case["Hk"], case["M"], case["N"], case["D"], case["dtype"],
+                      case["order"], case["std"])
+    _check(q, k, v, case["causal"], gpu_device)
+
+
+def test_rising_scores_force_the_redo_path(gpu_device):
+    """Keys whose scores rise by far more than the exponent range of a 16-bit P from tile to tile (a
+    known direction scaled up block by block): the step is redone against its true maximum."""
+    g = torch.Generator().manual_seed(9)
+    B, H, M, N, D = 1, 2, 300, 640, 128
+    q = torch.randn(B, H, M, D, generator=g)
+    k = torch.randn(B, H, N, D, generator=g)
+    v = torch.randn(B, H, N, D, generator=g)
+    ramp = torch.tensor([0.01, 1.0, 30.0, 0.01, 8.0, 0.01, 60.0, 1.0, 0.01, 20.0]).repeat_interleave(64).view(1, 1, N, 1)
+    k = k * ramp
+    for dtype in (torch.float16, torch.bfloat16):
+        for causal in (False, True):
+            _check(q.to(dtype), k.to(dtype), v.to(dtype), causal, gpu_device, sm_scale=0.5)
