@@ -2,9 +2,10 @@
 (src/flag_attn/flash.py:275-306): ``attention(q, k, v, causal=False, sm_scale=None, ...)`` on
 (batch, heads, sequence, head_dim) tensors of any strides with a unit innermost stride.
 
-Built here: the forward pass for fp16 / bf16, head_dim 64 or 128, grouped K/V heads, the causal flag
-for any qo_len / kv_len (bottom-right aligned, flash.py:53-54), ``sm_scale`` and the natural-log
-log normalizer (flash.py:503-506).  Not built: dropout, the total attention, head_dim 16 / 32 and the
+Built here: the forward pass for fp16 / bf16, head_dim 64 or 128 (16 and 32, which the reference also
+takes, flash.py:43, run through zero-padded copies of q, k, v at head_dim 64), grouped K/V heads, the
+causal flag for any qo_len / kv_len (bottom-right aligned, flash.py:53-54), ``sm_scale`` and the
+natural-log log normalizer (flash.py:503-506).  Not built: dropout, the total attention and the
 backward pass; a call that asks for one of them raises instead of computing something else.
 """
 from __future__ import annotations
@@ -46,8 +47,8 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
         raise NotImplementedError("flagattention_amd.flash.attention: dropout is not built")
     if return_total_attention:
         raise NotImplementedError("flagattention_amd.flash.attention: the total attention is not built")
-    if D not in (64, 128):
-        raise NotImplementedError(f"flagattention_amd.flash.attention: head_dim {D} is not built (64 or 128)")
+    if D not in (16, 32, 64, 128):
+        raise NotImplementedError(f"flagattention_amd.flash.attention: head_dim {D} is not built (16, 32, 64 or 128)")
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("q, k, v must share one of torch.float16 / torch.bfloat16")
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
@@ -60,6 +61,9 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     if M == 0 or N == 0 or B == 0:
         raise ValueError("empty q or k")
 
+    if D < 64:
+        # zero channels change neither Q K^T nor the first D columns of P V; sm_scale was fixed above from the true D
+        q, k, v = (torch.nn.functional.pad(t, (0, 64 - D)) for t in (q, k, v))
     q, k, v = _rows16(q), _rows16(k), _rows16(v)
     o = torch.empty_like(q)  # (the reference allocates the same way, flash.py:84-90)
     if not rows_aligned(o):
@@ -69,13 +73,15 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     p = _lib.FlashParams()
     p.q, p.k, p.v, p.out = (tensor_desc(t, True) for t in (q, k, v, o))
     p.log_normalizer = L.data_ptr() if L is not None else None
-    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = B, H, Hk, M, N, D
+    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = B, H, Hk, M, N, max(D, 64)
     p.dtype = p.out_dtype = DTYPE_CODE[q.dtype]
     p.causal = 1 if causal else 0
     p.sm_scale = float(sm_scale)
     lib = _lib.load()
     with torch.cuda.device(q.device):
         _lib.check(lib.sage_flash_attn_fwd(p, current_stream_ptr(q.device)), "sage_flash_attn_fwd")
+    if D < 64:
+        o = o[..., :D].contiguous()
     if return_log_normalizer:
         return o, L, None, None, None
     return o

@@ -117,7 +117,8 @@ int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out
  *   causal       non-zero: key n is visible to query m iff n <= m + (N - M) (flash.py:53-54, P_SEQ);
  *                a query that sees no key (M > N) yields a zero row and a log normalizer of -inf
  *   sm_scale     factor on Q K^T (the host passes 1/sqrt(head_dim) by default, flash.py:57-58)
- * head_dim must be 64 or 128 (the reference also takes 16 and 32); heads_q a multiple of heads_kv.
+ * head_dim must be 64 or 128 (the reference also takes 16 and 32: a caller pads those with zero
+ * channels, which changes neither Q K^T nor the first columns of P V); heads_q a multiple of heads_kv.
  */
 typedef struct sage_flash_params {
     sage_tensor q, k, v, out;

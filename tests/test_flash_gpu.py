@@ -114,7 +114,7 @@ def test_unbuilt_features_raise(gpu_device):
     with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q, k, v, return_total_attention=True)
     with pytest.raises(NotImplementedError):
-        flag_attn.flash_attention(q[..., :32], k[..., :32], v[..., :32])
+        flag_attn.flash_attention(q[..., :48], k[..., :48], v[..., :48])
     with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q.requires_grad_(), k, v)
     with pytest.raises(AssertionError):
@@ -176,3 +176,14 @@ def test_rising_scores_force_the_redo_path(gpu_device):
     for dtype in (torch.float16, torch.bfloat16):
         for causal in (False, True):
             _check(q.to(dtype), k.to(dtype), v.to(dtype), causal, gpu_device, sm_scale=0.5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", [(2, 4, 4, 1024, 1024, 32), (2, 4, 1, 1024, 1024, 16), (2, 4, 2, 1001, 1001, 32),
+                                           (1, 2, 1, 2048, 2058, 16)])
+def test_small_head_dims(B, Hq, Hk, M, N, D, causal, gpu_device):
+    """head_dim 16 and 32 (shapes of the reference's test list, tests/flag_attn/test_flash_attention.py:84-100)
+    run through zero-padded copies at head_dim 64; the default sm_scale is that of the true head_dim."""
+    q, k, v = _inputs(8, B, Hq, Hk, M, N, D, torch.float16)
+    o = _check(q, k, v, causal, gpu_device)
+    assert o.shape == q.shape and o.is_contiguous()
