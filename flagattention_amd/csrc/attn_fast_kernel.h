@@ -402,7 +402,20 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         };
         // The last DEFER of the 16 units wait for the MFMA phase (head_dim 64: that phase has half the
         // matrix instructions, so it takes a share of the exponentials to keep the two phases even).
-        sfor<16 - DEFER>(exp_unit);
+        // Where the row sums are taken is a measured choice per instance: in the shadow of the Q.K^T
+        // instructions everywhere (head_dim 128, int8: 10 % faster than here; 16-bit without hidden keys:
+        // 4 %), except in the 16-bit instance that hides keys, whose MFMA phase is the longer one (32 matrix
+        // instructions and the masking of the diagonal tiles): there they follow their exponentials (-4.5 %).
+        constexpr bool kSumsEarly = QB == 2 && CAUSAL && DEFER == 0;
+        sfor<16 - DEFER>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            exp_unit(uc);
+            if constexpr (kSumsEarly && u >= 2) lsum = PVT::dot2_ones(pf[(u - 2) >> 2], (u - 2) & 3, lsum);
+        });
+        if constexpr (kSumsEarly) {
+            lsum = PVT::dot2_ones(pf[3], 2, lsum);
+            lsum = PVT::dot2_ones(pf[3], 3, lsum);
+        }
         // A lane's 32 P of a step sum to less than kSumLimit, or the step is redone: so no P overflows the
         // 16-bit type (nor does a sum or a product with V come near the fp32 range), and a row whose scores
         // rise keeps its reference point within log2(kSumLimit) of its maximum.  Wave-wide decision; rare
@@ -410,7 +423,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // The sums are complete SUM_SLOTS matrix instructions into the phase; the wave vote on them is taken
         // there and only tested before the first P.V instruction, four matrix instructions later, so that
         // neither the last sum nor the compare is waited for (2-3 % on the causal and the 16-bit instances).
-        constexpr int SUM_SLOTS = (DEFER == 0 && QK_SLOTS >= 8) ? QK_SLOTS - 4 : QK_SLOTS;
+        constexpr int SUM_SLOTS = kSumsEarly ? -1 : (DEFER == 0 && QK_SLOTS >= 8) ? QK_SLOTS - 4 : QK_SLOTS;
         unsigned long long large = 0;
         auto redo_if_large = [&]() {
             if (large != 0) {
@@ -440,6 +453,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 });
             }
         };
+        if constexpr (kSumsEarly) large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));
         sc = step_scale(min(step + 1, nsteps - 1));
         __builtin_amdgcn_sched_barrier(0);
         // The first K fragments of the coming MFMA phase are requested before the barrier (their tile
@@ -469,7 +483,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 // row sums of P ride in the shadow of the Q.K^T instructions
                 sfor<16 - DEFER>([&](auto rc) {
                     constexpr int u = decltype(rc)::value;
-                    if constexpr (u * SUM_SLOTS / (16 - DEFER) == i) {
+                    if constexpr (!kSumsEarly && u * SUM_SLOTS / (16 - DEFER) == i) {
                         lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
                         asm volatile("" ::"v"(lsum));
                     }
@@ -481,7 +495,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             } else {
                 constexpr int j = i - QK_SLOTS, tp = j / F::DTILES, dt = j % F::DTILES;
                 if constexpr (j == 0) {
-                    if constexpr (SUM_SLOTS == QK_SLOTS) large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));
+                    if constexpr (!kSumsEarly && SUM_SLOTS == QK_SLOTS) large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));
                     redo_if_large();
                     __builtin_amdgcn_sched_barrier(0);
                 }
