@@ -187,3 +187,40 @@ def test_small_head_dims(B, Hq, Hk, M, N, D, causal, gpu_device):
     q, k, v = _inputs(8, B, Hq, Hk, M, N, D, torch.float16)
     o = _check(q, k, v, causal, gpu_device)
     assert o.shape == q.shape and o.is_contiguous()
+
+
+def test_side_stream_and_graph_replay(gpu_device):
+    """The library only enqueues kernels on the caller's stream: a side stream gives the same bits as the
+    default stream, and a captured graph of the call replays to them, with eager work between replays."""
+    import flag_attn
+
+    g = torch.Generator().manual_seed(41)
+    q, k, v = (torch.randn(2, 4, 520, 128, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
+
+    def call(qx):
+        return flag_attn.flash_attention(qx, k, v, True, return_log_normalizer=True)[:2]
+
+    want = [t.clone() for t in call(q)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = call(q)
+    side.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+
+    static_q = q.clone()
+    with torch.cuda.stream(side):
+        call(static_q)  # warm-up on the capture stream (allocator)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = call(static_q)
+    for rep in range(3):
+        src = q.flip(2) if rep == 1 else q
+        static_q.copy_(src)
+        expect = [t.clone() for t in call(src)]  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(captured, expect)), f"replay {rep}"
