@@ -224,3 +224,35 @@ def test_side_stream_and_graph_replay(gpu_device):
         graph.replay()
         torch.cuda.synchronize()
         assert all(torch.equal(a, b) for a, b in zip(captured, expect)), f"replay {rep}"
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_long_sequence_against_chunked_fp32(causal, gpu_device):
+    """N = 16384 (256 steps per workgroup; under the causal flag paired q-blocks of 4 and 256 steps): two
+    heads against an fp32 evaluation of the closed form done in row chunks on the GPU (plumbing only: the
+    closed form itself is the oracle's, pinned on the CPU), under the reference's acceptance rule with the
+    bf16 evaluation of the same chunks as the yardstick."""
+    import flag_attn
+
+    g = torch.Generator().manual_seed(77)
+    B, H, N, D = 1, 2, 16384, 128
+    q, k, v = (torch.randn(B, H, N, D, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
+    o, L, *_ = flag_attn.flash_attention(q, k, v, causal, return_log_normalizer=True)
+    torch.cuda.synchronize()
+    scale = 1.0 / math.sqrt(D)
+    worst = yard = worst_l = 0.0
+    for m0 in range(0, N, 2048):
+        rows = slice(m0, m0 + 2048)
+        s = (q[:, :, rows].float() @ k.float().transpose(2, 3)) * scale
+        s16 = ((q[:, :, rows] @ k.transpose(2, 3)) * scale).float()
+        if causal:
+            vis = torch.arange(m0, m0 + 2048, device=gpu_device).unsqueeze(-1) >= torch.arange(N, device=gpu_device)
+            s = s.masked_fill(~vis, float("-inf"))
+            s16 = s16.masked_fill(~vis, float("-inf"))
+        ref = torch.softmax(s, dim=-1) @ v.float()
+        o16 = (torch.softmax(s16, dim=-1).to(torch.bfloat16) @ v).float()
+        worst = max(worst, (o[:, :, rows].float() - ref).abs().max().item())
+        yard = max(yard, (o16 - ref).abs().max().item())
+        worst_l = max(worst_l, (L[:, :, rows] - torch.logsumexp(s, dim=-1)).abs().max().item())
+    assert worst <= 2 * yard + 1e-5, (worst, yard)
+    assert worst_l <= 2e-3, worst_l
