@@ -475,3 +475,25 @@ def test_benchmark_rows_on_a_small_shape(gpu_device):
     assert row["error_msg"] is None and row["latency"] > 0 and row["tflops"] > 0
     if row["base_miss_reason"] is None:
         assert row["accuracy"] >= 0.99 and row["relative_l2"] <= 0.05 and row["speedup"] > 0
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_extreme_int8_values(d, gpu_device):
+    """Largest dot products int8 operands can produce (-128 * -128 * head_dim = 2^21 at head_dim 128, and
+    the most negative one): the Q.K^T accumulators are read as floats through a 1.5 * 2^23 bias, which holds
+    for |dot| < 2^22; caller-made int8 tensors may contain -128 although the quantizer never writes it."""
+    m, n = 160, 192
+    g = torch.Generator().manual_seed(17)
+    q8 = torch.full((1, 2, m, d), -128, dtype=torch.int8)
+    k8 = torch.full((1, 2, n, d), -128, dtype=torch.int8)
+    k8[:, :, 1::3] = 127       # most negative products
+    k8[:, :, 2::3] = torch.randint(-128, 128, (1, 2, len(range(2, n, 3)), d), generator=g, dtype=torch.int8)
+    q8[:, :, ::5] = torch.randint(-128, 128, (1, 2, len(range(0, m, 5)), d), generator=g, dtype=torch.int8)
+    qs = torch.full((1, 2, 2), 3.0e-4)
+    ks = torch.full((1, 2, 3), 2.0e-3)
+    v = torch.randn(1, 2, n, d, generator=g).to(torch.bfloat16)
+    for causal in (False, True):
+        o, lse = _run(gpu_device, q8, qs, k8, ks, v, causal=causal, return_lse=True, output_dtype=torch.float32)
+        expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, causal=causal)
+        _gate(o, expected)
+        torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-5)
