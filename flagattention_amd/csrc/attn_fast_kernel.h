@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int DEFER = D == 64 ? 4 : 0;                   // exponential units moved into the MFMA phase
+    constexpr int DEFER = (D == 64 && INT8) ? 4 : 0;        // exponential units moved into the MFMA phase (measured per instance)
     constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
     constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
