@@ -2,6 +2,35 @@
 // over head_dim, the 16-bit type of V and P, whether keys can be hidden, and the width of Q and K
 // elements.  Included by the two translation units that instantiate it: attn_fwd_fast.hip (int8 Q, K:
 // SageAttention) and flash_fwd.hip (16-bit Q, K: dense attention).
+//
+// Per workgroup: 8 waves x 32 query rows (two q_scale blocks of the int8 path, so that every K/V tile
+// staged in LDS serves 256 rows); per step: 64 keys (one k_scale block).  Every wave computes the transposed
+// products S^T = K.Q^T (8 x v_mfma_i32_32x32x32_i8, or 16 x v_mfma_f32_32x32x16 for 16-bit Q and K, at
+// head_dim 128) and O^T += V^T.P^T (16 x v_mfma_f32_32x32x16)
+// so that a lane owns one query row and P never leaves registers.
+//
+// * K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4, 16 bytes per
+//   lane), four tiles of each resident: tile t lives in buffer t % 4 and is fetched during the VALU
+//   phase two (V) or three (K) steps before the step that multiplies with it.  LDS rows are
+//   unpadded; bank conflicts are avoided by an XOR swizzle of the 16-byte chunks of a row, applied
+//   on the global-address side of the load and undone by the fragment reads.
+// * V is read with ds_read_b64_tr_b16, which hands each lane four consecutive keys of one channel:
+//   exactly the A operand of the P.V MFMA, with no shuffling instructions.
+// * Every wave alternates between a VALU phase (exponentials of step j) and an MFMA phase (Q.K^T of
+//   step j+1 and P.V of step j back to back, with the row sums of P riding in the shadow of the
+//   matrix instructions).  The two waves that share a SIMD
+//   run half a step apart, so the matrix core and the VALU are both kept busy; phases are
+//   separated by workgroup barriers (two per step).
+// * (int8) The int32 Q.K^T accumulators start from the bit pattern of 1.5 * 2^23, so their bits ARE the
+//   float kBias + dot and no int -> float conversion is issued; the two score register sets swap
+//   roles every step (the loop body exists for both parities).
+// * No row maximum is taken per step: exponentials use the reference point the row already has
+//   (the maximum of its first tile to begin with), and a step whose row sums come out large is
+//   redone against its true maximum before any P.V instruction of it has been issued.  The row
+//   sums are needed anyway, so the common step pays nothing for the check but a compare.
+// * 16-bit outputs are transposed through LDS and written as whole rows.
+// * Under the causal flag a workgroup takes two q-blocks of its head (the longest remaining and the
+//   shortest), so that all workgroups of a launch run the same number of steps.
 #pragma once
 #include <utility>
 
