@@ -48,6 +48,9 @@ template <> struct PV<__bf16> {
     static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ v4f mfma16(vec a, vec b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
     // acc + p[2c] + p[2c+1]
     static __device__ __forceinline__ float dot2_ones(vec p, int c, float acc) {
         typedef __bf16 v2 __attribute__((ext_vector_type(2)));
@@ -60,6 +63,9 @@ template <> struct PV<_Float16> {
     typedef f16x8 vec;
     static __device__ __forceinline__ v16f mfma(vec a, vec b, v16f c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ v4f mfma16(vec a, vec b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ float dot2_ones(vec p, int c, float acc) {
         typedef _Float16 v2 __attribute__((ext_vector_type(2)));

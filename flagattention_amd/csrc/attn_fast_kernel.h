@@ -260,6 +260,18 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "s"(INT8 ? kBiasBits : 0));
         bias16[i] = b;
     }
+    // Row sums of P by the matrix core: one 16x16x32 instruction per 16-key slice multiplies a 0/1 pattern
+    // with the slice's P^T registers as they are.  Read as a 32 x 16 B operand, those registers hold four
+    // groups of eight keys: (rows 0-15 | rows 16-31) x (keys 0-7 | keys 8-15) of the slice; output rows
+    // 0-3 and 8-11 add the two groups of rows 0-15, output rows 4-7 and 12-15 those of rows 16-31, which
+    // is where the lanes that own those query rows read their results.  Every lane ends up with the sum
+    // over all 16 keys of its own row (both halves), in four equal registers.
+    vec16 sum_pattern;
+    {
+        const VT c = (((lane >> 4) & 1) == ((lane >> 2) & 1)) ? (VT)1.0f : (VT)0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) sum_pattern[e] = c;
+    }
     auto qk_mfma = [](v4i kf, v4i q, v16i acc) {
         if constexpr (INT8) {
             return __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, q, acc, 0, 0, 0);
@@ -295,6 +307,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
     constexpr int DEFER = (D == 64 && INT8) ? 4 : 0;        // exponential units moved into the MFMA phase (measured per instance)
+    constexpr bool kWholeRowSums = QB == 2 && !CAUSAL;      // row sums by the matrix core: every lane holds its whole row's sum
     constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
     constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
     static_assert(KDIST <= QK_SLOTS && VDIST < QK_SLOTS && 16 % QK_SLOTS == 0, "slot plan");
@@ -452,7 +465,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // The sums are complete SUM_SLOTS matrix instructions into the phase; the wave vote on them is taken
         // there and only tested before the first P.V instruction, four matrix instructions later, so that
         // neither the last sum nor the compare is waited for (2-3 % on the causal and the 16-bit instances).
+        // ... and in the 16-bit instance without hidden keys the matrix core takes them (sum_pattern above): four
+        // cheap matrix instructions instead of 16 v_dot2 on an issue port that the 32 matrix instructions of
+        // its step already load (-5 %; neutral for the int8 instances, which keep v_dot2 and half-row sums).
+        constexpr bool kMfmaSums = kWholeRowSums;
         constexpr int SUM_SLOTS = kSumsEarly ? -1 : (DEFER == 0 && QK_SLOTS >= 8) ? QK_SLOTS - 4 : QK_SLOTS;
+        v4f sum4 = {0.0f, 0.0f, 0.0f, 0.0f};
         unsigned long long large = 0;
         auto redo_if_large = [&]() {
             if (large != 0) {
@@ -480,6 +498,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                     exp_unit(uc);
                     lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
                 });
+                if constexpr (kMfmaSums) lsum += __shfl_xor(lsum, 32);  // this instance keeps whole-row sums in every lane
             }
         };
         if constexpr (kSumsEarly) large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));
@@ -510,14 +529,26 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 if constexpr (i + KDIST < QK_SLOTS) read_k(IC<i + KDIST>{});
                 if constexpr (i >= QK_SLOTS - VDIST) read_v(IC<i - (QK_SLOTS - VDIST)>{});
                 // row sums of P ride in the shadow of the Q.K^T instructions
-                sfor<16 - DEFER>([&](auto rc) {
-                    constexpr int u = decltype(rc)::value;
-                    if constexpr (!kSumsEarly && u * SUM_SLOTS / (16 - DEFER) == i) {
-                        lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
-                        asm volatile("" ::"v"(lsum));
+                if constexpr (kMfmaSums) {
+                    if constexpr (i < 4) {  // one per slot, behind the first four Q.K^T instructions
+                        if constexpr (i == 0) sum4 = PVT::mfma16(sum_pattern, pf[0], v4f{0.0f, 0.0f, 0.0f, 0.0f});
+                        else sum4 = PVT::mfma16(sum_pattern, pf[i], sum4);
                     }
-                });
-                if constexpr (i == SUM_SLOTS - 1 && SUM_SLOTS < QK_SLOTS) {
+                    if constexpr (i == QK_SLOTS - 2) {  // the four sum instructions have long finished
+                        lsum = sum4[0];
+                        large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));  // also set for inf and NaN
+                        asm volatile("" ::"s"(large));
+                    }
+                } else {
+                    sfor<16 - DEFER>([&](auto rc) {
+                        constexpr int u = decltype(rc)::value;
+                        if constexpr (!kSumsEarly && u * SUM_SLOTS / (16 - DEFER) == i) {
+                            lsum = PVT::dot2_ones(pf[u >> 2], u & 3, lsum);
+                            asm volatile("" ::"v"(lsum));
+                        }
+                    });
+                }
+                if constexpr (!kMfmaSums && i == SUM_SLOTS - 1 && SUM_SLOTS < QK_SLOTS) {
                     large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));  // also set for inf and NaN
                     asm volatile("" ::"s"(large));
                 }
@@ -571,8 +602,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     if (wave < kFastWaves / 2) __syncthreads();
     __syncthreads();  // nobody reads or fills a K/V tile any more: the LDS is free for the output
     // ---- epilogue: O = O^T / l, lse = log2(l) + m
+    // (the instances that take the row sums with v_dot2 hold half a row's sum per lane)
     const float l_o = __shfl_xor(l_i, 32);
-    const float l_tot = half ? (l_o + l_i) : (l_i + l_o);
+    const float l_tot = kWholeRowSums ? l_i : half ? (l_o + l_i) : (l_i + l_o);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;  // l = 0: a row that saw no key; its output is 0, its lse -inf
     const int64_t obase_wave = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)(m0 + 32 * wave) * a.os_n;
     if (a.out_dt != SAGE_F32) {
