@@ -497,3 +497,30 @@ def test_extreme_int8_values(d, gpu_device):
         expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, causal=causal)
         _gate(o, expected)
         torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_repeated_calls_are_bit_identical(causal, gpu_device):
+    """No atomics and a fixed order of accumulation: 20 calls on the same inputs give the same bits (a tile
+    read before it has landed, or a buffer refilled too early, would show up here as a difference)."""
+    from flag_attn import sage_attention as sa
+    import flag_attn
+
+    g = torch.Generator().manual_seed(23)
+    q, k, v = (torch.randn(2, 8, 1536, 128, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
+    q8, qs, k8, ks = sa.per_block_int8(q, k, smooth_k=True)
+    first = sa.sage_attention(q8, k8, v, qs, ks, output_dtype=torch.bfloat16, causal=causal, return_lse=True)
+    dense_first = flag_attn.flash_attention(q, k, v, causal, return_log_normalizer=True)[:2]
+    for _ in range(20):
+        again = sa.sage_attention(q8, k8, v, qs, ks, output_dtype=torch.bfloat16, causal=causal, return_lse=True)
+        assert torch.equal(again[0], first[0]) and torch.equal(again[1], first[1])
+        dense_again = flag_attn.flash_attention(q, k, v, causal, return_log_normalizer=True)[:2]
+        assert torch.equal(dense_again[0], dense_first[0]) and torch.equal(dense_again[1], dense_first[1])
+    for d, dt in ((64, torch.float16),):
+        q2, k2, v2 = (torch.randn(2, 8, 1100, d, generator=g).to(dt).to(gpu_device) for _ in range(3))
+        a8, as_, b8, bs = sa.per_block_int8(q2, k2)
+        first = sa.sage_attention(a8, b8, v2, as_, bs, output_dtype=dt, causal=causal)[0]
+        dense_first = flag_attn.flash_attention(q2, k2, v2, causal)
+        for _ in range(20):
+            assert torch.equal(sa.sage_attention(a8, b8, v2, as_, bs, output_dtype=dt, causal=causal)[0], first)
+            assert torch.equal(flag_attn.flash_attention(q2, k2, v2, causal), dense_first)
