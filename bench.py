@@ -41,6 +41,7 @@ MEASURED_ATTN_TRAFFIC_BYTES = {"c2": 402.9e6}
 
 WORKLOADS = {
     # name: (B, H, N, D, dtype, layout, causal, description)
+    "c1": (1, 2, 256, 64, torch.float16, "HND", False, "cpu_plumbing_B1_H2_N256_D64_fp16_HND_noncausal_smoothk"),
     "c2": (4, 32, 4096, 128, torch.bfloat16, "HND", False, "llama_prefill_B4_H32_N4096_D128_bf16_HND_noncausal_smoothk"),
     "c3": (2, 32, 8192, 128, torch.bfloat16, "NHD", True, "causal_prefill_B2_H32_N8192_D128_bf16_NHD_causal_smoothk"),
     "c4": (8, 16, 2048, 64, torch.float16, "HND", False, "outlier_B8_H16_N2048_D64_fp16_HND_noncausal"),
@@ -58,8 +59,8 @@ def make_inputs(name, device):
         k = k + 2.0 * torch.randn((1, 1, h, d), generator=g)
     if name == "c4":
         idx = torch.randperm(h * d, generator=g)[:10]
-        for t in (q, k):
-            t.permute(0, 2, 1, 3).reshape(b, n, h * d)[..., idx] *= 20
+        for t in (q, k):  # 1 % of the (head, channel) pairs carry x20 outliers, the same pairs in Q and K
+            t[:, idx // d, :, idx % d] *= 20
         v = torch.rand(shape, generator=g) * 2 - 1
     else:
         v = torch.randn(shape, generator=g)

@@ -41,7 +41,7 @@ extern "C" int sage_per_block_int8(const sage_quant_params* p, void* stream) {
                     (long long)p->blkk * p->head_dim);
     if (p->q.ptr && (!p->q_int8.ptr || !p->q_scale)) return fail(SAGE_E_INVALID, "sage_per_block_int8: null Q output");
     if (p->k.ptr && (!p->k_int8.ptr || !p->k_scale)) return fail(SAGE_E_INVALID, "sage_per_block_int8: null K output");
-    if (p->km.ptr) {
+    if (p->km.ptr && p->k.ptr) {  // km belongs to K: a call that quantizes Q only ignores it
         if (!float_dtype_ok(p->km_dtype) || !float_dtype_ok(p->diff_dtype))
             return fail(SAGE_E_INVALID, "sage_per_block_int8: bad km_dtype/diff_dtype");
         if (p->in_dtype == SAGE_F32 && p->diff_dtype != SAGE_F32)

@@ -300,106 +300,6 @@ def test_seeded_shape_sweep(case, gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
 
 
-def _gpu_dequant_reference(q8, k8, v, qs, ks, heads, causal=False):
-    """fp32 softmax attention of the dequantized operands for a few (batch, head) pairs, on the GPU
-    (the same closed form as the oracle's attention_dequant; used where the CPU would take minutes)."""
-    outs = []
-    for b, h in heads:
-        hk = h // (q8.shape[1] // k8.shape[1])
-        q = q8[b, h].float() * qs[b, h].repeat_interleave(128)[: q8.shape[2], None]
-        k = k8[b, hk].float() * ks[b, hk].repeat_interleave(64)[: k8.shape[2], None]
-        s = (q @ k.T) * math.log(2.0)
-        if causal:
-            m, n = s.shape
-            s = s.masked_fill(~(torch.arange(n, device=s.device)[None] <= torch.arange(m, device=s.device)[:, None] + (n - m)),
-                              float("-inf"))
-        outs.append(torch.softmax(s, dim=-1) @ v[b, hk].float())
-    return torch.stack(outs)
-
-
-def test_north_star_config_full_size(gpu_device):
-    """B4 H32 N4096 D128 bf16 HND non-causal, K smoothing on: CPU oracle on two heads, GPU fp32
-    closed form on eight, benchmark-style gate against SDPA on the unquantized inputs."""
-    from flag_attn import sage_attention as sa
-
-    g = torch.Generator().manual_seed(42)
-    q, k, v = (torch.randn(4, 32, 4096, 128, generator=g).to(torch.bfloat16) for _ in range(3))
-    qd, kd, vd = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
-    q8, qs, k8, ks = sa.per_block_int8(qd, kd, smooth_k=True)
-    o, lse = sa.sage_attention(q8, k8, vd, qs, ks, output_dtype=torch.bfloat16, return_lse=True)
-    torch.cuda.synchronize()
-    heads = [(0, 0), (3, 31)]
-    for b, h in heads:
-        sl = (slice(b, b + 1), slice(h, h + 1))
-        exp, exp_lse = C.attention_blockwise(q8[sl].cpu(), k8[sl].cpu(), v[sl], qs[sl].cpu(), ks[sl].cpu())
-        _gate(o[sl], exp, f"head {b},{h}")
-        torch.testing.assert_close(lse[sl].cpu(), exp_lse, atol=2e-3, rtol=1e-4)
-    heads = [(b, h) for b in range(4) for h in (5, 20)]
-    ref = _gpu_dequant_reference(q8, k8, vd, qs, ks, heads)
-    got = torch.stack([o[b, h] for b, h in heads])
-    _gate(got, ref, "gpu closed form")
-    base = torch.nn.functional.scaled_dot_product_attention(qd[:1], kd[:1], vd[:1])
-    cos, rel, _ = O.accuracy_metrics(o[:1].cpu(), base.cpu())
-    assert cos >= 0.99 and rel <= 0.05  # benchmark/test_sage_attention_benchmark.py:174-177
-
-
-def test_causal_nhd_config_shape(gpu_device):
-    """B2 H32 N8192 D128 NHD bf16 causal, K = N(0,1) + per-channel offset N(0,4) (batch cut to 1)."""
-    from flag_attn import sage_attention as sa
-
-    g = torch.Generator().manual_seed(42)
-    b, n, h, d = 1, 8192, 32, 128
-    q = torch.randn(b, n, h, d, generator=g).to(torch.bfloat16)
-    k = (torch.randn(b, n, h, d, generator=g) + 2.0 * torch.randn(1, 1, h, d, generator=g)).to(torch.bfloat16)
-    v = torch.randn(b, n, h, d, generator=g).to(torch.bfloat16)
-    qd, kd, vd = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
-    q8, qs, k8, ks = sa.per_block_int8(qd, kd, tensor_layout="NHD", smooth_k=True)
-    o, _ = sa.sage_attention(q8, k8, vd, qs, ks, tensor_layout="NHD", output_dtype=torch.bfloat16, causal=True)
-    heads = [(0, 0), (0, 17), (0, 31)]
-    ref = _gpu_dequant_reference(q8.transpose(1, 2), k8.transpose(1, 2), vd.transpose(1, 2), qs, ks, heads, causal=True)
-    got = torch.stack([o[bb, :, hh] for bb, hh in heads])
-    _gate(got, ref)
-    base = torch.nn.functional.scaled_dot_product_attention(
-        qd.transpose(1, 2)[:, :4], kd.transpose(1, 2)[:, :4], vd.transpose(1, 2)[:, :4], is_causal=True)
-    cos, rel, _ = O.accuracy_metrics(o.transpose(1, 2)[:, :4].cpu(), base.cpu())
-    assert cos >= 0.99 and rel <= 0.05
-
-
-def test_outlier_d64_config_shape(gpu_device):
-    """B8 H16 N2048 D64 fp16, 1% outlier channels x20 in Q and K, V ~ U(-1,1) (batch cut to 2)."""
-    from flag_attn import sage_attention as sa
-
-    g = torch.Generator().manual_seed(42)
-    b, h, n, d = 2, 16, 2048, 64
-    q = torch.randn(b, h, n, d, generator=g)
-    k = torch.randn(b, h, n, d, generator=g)
-    idx = torch.randperm(h * d, generator=g)[:10]
-    for t in (q, k):
-        t.permute(0, 2, 1, 3).reshape(b, n, h * d)[..., idx] *= 20
-    v = torch.rand(b, h, n, d, generator=g) * 2 - 1
-    q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
-    q8, qs, k8, ks = sa.per_block_int8(q.to(gpu_device), k.to(gpu_device))
-    o, lse = sa.sage_attention(q8, k8, v.to(gpu_device), qs, ks, return_lse=True)
-    exp, exp_lse = C.attention_blockwise(q8[:1, :4].cpu(), k8[:1, :4].cpu(), v[:1, :4], qs[:1, :4].cpu(), ks[:1, :4].cpu())
-    _gate(o[:1, :4], exp)
-    torch.testing.assert_close(lse[:1, :4].cpu(), exp_lse, atol=2e-3, rtol=1e-4)
-    heads = [(bb, hh) for bb in range(b) for hh in (3, 9, 15)]
-    ref = _gpu_dequant_reference(q8, k8, v.to(gpu_device), qs, ks, heads)
-    _gate(torch.stack([o[bb, hh] for bb, hh in heads]), ref)
-
-
-def test_long_sequence_config_shape(gpu_device):
-    """B1 H24 N32768 D128 bf16 non-causal, K smoothing on (heads cut to 4)."""
-    from flag_attn import sage_attention as sa
-
-    g = torch.Generator().manual_seed(42)
-    q, k, v = (torch.randn(1, 4, 32768, 128, generator=g).to(torch.bfloat16).to(gpu_device) for _ in range(3))
-    q8, qs, k8, ks = sa.per_block_int8(q, k, smooth_k=True)
-    o, _ = sa.sage_attention(q8, k8, v, qs, ks, output_dtype=torch.bfloat16)
-    ref = _gpu_dequant_reference(q8, k8, v, qs, ks, [(0, 1)])
-    _gate(o[0, 1][None], ref)
-
-
 def test_sageattn_wrapper_lse(gpu_device):
     from flag_attn.sage_attention import sageattn
 

@@ -36,6 +36,38 @@ def test_struct_layouts_match_header():
     assert ctypes.sizeof(_lib.SageTensor) == 32
     assert ctypes.sizeof(_lib.QuantParams) == 5 * 32 + 2 * 8 + 6 * 8 + 6 * 4
     assert ctypes.sizeof(_lib.AttnParams) == 4 * 32 + 4 * 8 + 4 * 8 + 6 * 8 + 4 * 4
+    assert ctypes.sizeof(_lib.FlashParams) == 4 * 32 + 8 + 6 * 8 + 3 * 4 + 4
+    # field offsets, compiled from the header itself
+    import shutil
+    import subprocess
+    import tempfile
+
+    if shutil.which("gcc") is None:
+        pytest.skip("needs gcc for the offsetof check")
+    fields = {
+        "sage_quant_params": (_lib.QuantParams, ["q", "k", "km", "q_int8", "k_int8", "q_scale", "k_scale", "batch",
+                                                 "head_dim", "in_dtype", "km_dtype", "diff_dtype", "blkq", "blkk", "q_mul"]),
+        "sage_attn_params": (_lib.AttnParams, ["q", "out", "q_scale", "k_scale", "lse", "mask", "mask_stride_b",
+                                               "mask_stride_n", "batch", "head_dim", "v_dtype", "out_dtype", "mask_kind", "causal"]),
+        "sage_flash_params": (_lib.FlashParams, ["q", "out", "log_normalizer", "batch", "head_dim", "dtype", "out_dtype",
+                                                 "causal", "sm_scale"]),
+    }
+    lines = ['#include <stddef.h>', '#include <stdio.h>', f'#include "{HEADER}"', "int main(void) {"]
+    for cname, (_, names) in fields.items():
+        lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
+        for n in names:
+            lines.append(f'printf("{cname}.{n} %zu\\n", offsetof({cname}, {n}));')
+    lines.append("return 0; }")
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "off.c")
+        open(src, "w").write("\n".join(lines))
+        subprocess.run(["gcc", "-o", os.path.join(tmp, "off"), src], check=True)
+        out = subprocess.run([os.path.join(tmp, "off")], capture_output=True, text=True, check=True).stdout
+    seen = dict(line.rsplit(" ", 1) for line in out.splitlines())
+    for cname, (cls, names) in fields.items():
+        assert int(seen[cname]) == ctypes.sizeof(cls), cname
+        for n in names:
+            assert int(seen[f"{cname}.{n}"]) == getattr(cls, n).offset, f"{cname}.{n}"
 
 
 def test_validation_without_gpu_work():

@@ -264,3 +264,31 @@ def test_flash_oracle_causal_alignment_brute_force(m, n):
     torch.testing.assert_close(lse.double()[fin], blse[fin], atol=1e-5, rtol=1e-6)
     if m > n:
         assert float(o[:, :, : m - n].abs().max()) == 0.0
+
+
+def test_accuracy_metrics_known_answers():
+    """The gate's own yardstick (cosine, relative L2, max-abs) on vectors whose answers are known by hand."""
+    e1 = torch.tensor([3.0, 0.0, 0.0, 0.0])
+    e2 = torch.tensor([0.0, 4.0, 0.0, 0.0])
+    cos, rel, max_abs = O.accuracy_metrics(e1, e2)  # orthogonal
+    assert abs(cos) < 1e-12 and abs(rel - 5.0 / 4.0) < 1e-12 and max_abs == 4.0
+    cos, rel, max_abs = O.accuracy_metrics(-e1, e1)  # opposite
+    assert abs(cos + 1.0) < 1e-12 and abs(rel - 2.0) < 1e-12 and max_abs == 6.0
+    cos, rel, max_abs = O.accuracy_metrics(2.0 * e1, e1)  # parallel, twice as long: the cosine cannot see it
+    assert abs(cos - 1.0) < 1e-12 and abs(rel - 1.0) < 1e-12 and max_abs == 3.0
+    # 3-4-5 triangle: cos = 3/5; |a - e| = 4 against |e| = 3
+    cos, rel, max_abs = O.accuracy_metrics(torch.tensor([3.0, 4.0]), torch.tensor([3.0, 0.0]))
+    assert abs(cos - 0.6) < 1e-12 and abs(rel - 4.0 / 3.0) < 1e-12 and max_abs == 4.0
+    # one outlier in a long vector: max-abs is taken over EVERY element, the cosine / L2 over the strided sample
+    # (benchmark/test_sage_attention_benchmark.py:136-149: stride = ceil(numel / max_elements))
+    a = torch.ones(10)
+    e = torch.ones(10)
+    a[7] = 9.0
+    cos, rel, max_abs = O.accuracy_metrics(a, e, max_elements=4)  # stride 3: elements 0, 3, 6, 9
+    assert max_abs == 8.0 and abs(cos - 1.0) < 1e-12 and rel == 0.0
+    a[6] = 3.0
+    cos, rel, max_abs = O.accuracy_metrics(a, e, max_elements=4)  # sample (1,1,3,1) against (1,1,1,1)
+    assert abs(cos - 6.0 / (math.sqrt(12.0) * 2.0)) < 1e-12 and abs(rel - 2.0 / 2.0) < 1e-12 and max_abs == 8.0
+    # shapes are flattened, 16-bit inputs are compared in fp32 / fp64
+    cos, rel, max_abs = O.accuracy_metrics(torch.ones(2, 3, dtype=torch.bfloat16), torch.full((2, 3), 1.5))
+    assert abs(cos - 1.0) < 1e-12 and abs(rel - 1.0 / 3.0) < 1e-12 and max_abs == 0.5
