@@ -10,6 +10,7 @@ ABI_VERSION = 2
 
 SAGE_F16, SAGE_BF16, SAGE_F32 = 0, 1, 2
 MASK_NONE, MASK_BOOL, MASK_F32 = 0, 1, 2
+K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES = 8 * 1024 * 1024
 
 c_i64 = ctypes.c_int64
 c_i32 = ctypes.c_int32
@@ -60,6 +61,7 @@ EXPORTS = (
     "sage_flash_attn_fwd",
     "sage_k_mean",
     "sage_k_mean_workspace_bytes",
+    "sage_k_mean_noalloc",
     "sage_hip_last_error",
     "sage_hip_abi_version",
 )
@@ -94,6 +96,9 @@ def load():
     lib.sage_k_mean.argtypes = [ctypes.POINTER(SageTensor), c_i32, ctypes.c_void_p, c_i32, c_i64, c_i64, c_i64,
                                 c_i64, ctypes.c_void_p, ctypes.c_void_p]
     lib.sage_k_mean.restype = ctypes.c_int
+    lib.sage_k_mean_noalloc.argtypes = [ctypes.POINTER(SageTensor), c_i32, ctypes.c_void_p, c_i32, c_i64, c_i64, c_i64,
+                                        c_i64, ctypes.c_void_p]
+    lib.sage_k_mean_noalloc.restype = ctypes.c_int
     if lib.sage_hip_abi_version() != ABI_VERSION:
         raise ImportError(f"{LIB_PATH}: ABI version {lib.sage_hip_abi_version()} != {ABI_VERSION}; rebuild it")
     _lib = lib

@@ -65,6 +65,27 @@ extern "C" int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, 
                         (hipStream_t)stream);
 }
 
+extern "C" int sage_k_mean_noalloc(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out_dtype, int64_t batch,
+                                   int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* stream) {
+    if (!k || !k->ptr || !km_out) return fail(SAGE_E_INVALID, "sage_k_mean_noalloc: null pointer");
+    if (!float_dtype_ok(k_dtype) || !float_dtype_ok(out_dtype))
+        return fail(SAGE_E_INVALID, "sage_k_mean_noalloc: bad dtype");
+    if (batch <= 0 || heads_kv <= 0 || kv_len <= 0 || head_dim <= 0)
+        return fail(SAGE_E_INVALID, "sage_k_mean_noalloc: sizes must be positive");
+    // (each factor bounded first, so the product below cannot overflow)
+    const int64_t lim = SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES;
+    if (batch > lim || heads_kv > lim || kv_len > (lim << 6) || head_dim > lim ||
+        batch * heads_kv > lim || batch * heads_kv * ((kv_len + 63) / 64) > lim ||
+        sage_k_mean_workspace_bytes(batch, heads_kv, kv_len, head_dim) > lim)
+        return fail(SAGE_E_UNSUPPORTED,
+                    "sage_k_mean_noalloc: batch %lld x heads %lld x ceil(kv_len %lld / 64) x head_dim %lld fp32 partials "
+                    "exceed the built-in %lld-byte scratch; use sage_k_mean with a workspace",
+                    (long long)batch, (long long)heads_kv, (long long)kv_len, (long long)head_dim, (long long)lim);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return launch_kmean(*k, k_dtype, km_out, out_dtype, batch, heads_kv, kv_len, head_dim, ws, (hipStream_t)stream);
+}
+
 extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
     if (!p) return fail(SAGE_E_INVALID, "sage_attn_fwd: null params");
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr || !p->out.ptr || !p->q_scale || !p->k_scale)

@@ -10,12 +10,23 @@
 // HBM-bound: one workgroup per [BLK, D] block reads the block once (16-byte loads, coalesced
 // along head_dim), keeps it in registers as fp32, reduces max|x| with wave shuffles plus one LDS
 // step, and writes 8-byte int8 groups.  Algorithmic traffic: in_bytes + 1 byte per element.
+#include <mutex>
+
 #include "common.h"
 
 namespace sage {
 namespace {
 
 constexpr int kThreads = 256;
+
+// Chunk partials of the K mean for the entry point that takes no workspace (sage_k_mean_noalloc).  Each GPU
+// holds its own copy of this array, at its own address, until the process ends; the name below is a host-side
+// handle only, so every use goes through the address hipGetSymbolAddress returns for the current device.
+constexpr size_t kScratchBytes = SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};  // per device: address of that device's copy of `scratch`
 
 struct QuantArgs {
     const void* x;
@@ -366,6 +377,24 @@ __global__ __launch_bounds__(kThreads) void k_mean_final_kernel(KMeanArgs a, int
 }
 
 }  // namespace
+
+// Address of the current device's copy of the static scratch array (looked up once per device).
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SAGE_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(SAGE_E_UNSUPPORTED, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(SAGE_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SAGE_OK;
+}
 
 int launch_quant(const sage_quant_params& p, hipStream_t stream) {
     const int esz = dtype_bytes(p.in_dtype);

@@ -106,6 +106,21 @@ int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out
                 int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* workspace, void* stream);
 
 /*
+ * sage_k_mean without a workspace argument and without any allocation: no counterpart in the reference.
+ * It is for callers that cannot allocate device memory around the call (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the chunk partials go to a fixed array inside the
+ * library's device image, SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES per GPU, held until the process ends.
+ * Same arguments, order of additions and result bits as sage_k_mean.  A call whose
+ * sage_k_mean_workspace_bytes(...) exceeds the maximum is rejected with SAGE_E_UNSUPPORTED (nothing is
+ * launched).  All calls on one GPU share that GPU's array: two calls that may run concurrently on one GPU
+ * (different streams, different threads) race; calls ordered on one stream do not.  Nothing needs to start
+ * from zero: every partial a call reads was written by that call.
+ */
+#define SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES (8 * 1024 * 1024)
+int sage_k_mean_noalloc(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out_dtype, int64_t batch,
+                        int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* stream);
+
+/*
  * Dense attention forward on 16-bit Q, K, V: replaces the forward launch of FlagAttention's
  * flash_attention (src/flag_attn/flash.py:37-180 host, :346-510 kernel) for the calls that need no
  * dropout, no total attention and no gradient:  O = softmax(sm_scale * Q K^T [+ causal]) V.
