@@ -142,6 +142,29 @@ def test_upstream_vendor_package_resolves_to_this_build():
         assert fn is want
 
 
+def test_upstream_vendor_package_through_the_reference_registry():
+    """What the reference's own registry (op_registry.py:17-60) returns for the shipped ``_amd`` package:
+    recorded by tests/golden/make_registry_golden.py, checked against this build's functions; where the
+    reference checkout is present the resolution is also done live."""
+    import json
+
+    from flagattention_amd import sage_attention as sa
+
+    golden = json.load(open(os.path.join(ROOT, "tests", "golden", "registry_golden.json")))
+    want = {"sage_attention": sa.forward, "sage_attention_forward": sa.forward, "sage_attention_per_block_int8": sa.per_block_int8}
+    for name, fn in want.items():
+        assert golden[name] == [fn.__module__, fn.__qualname__], name
+    assert golden["flash_attention (not declared: generic math.sqrt)"] == ["math", "sqrt"]
+    sys_path_entry = os.path.join(ROOT, "tests", "golden")
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("make_registry_golden", os.path.join(sys_path_entry, "make_registry_golden.py"))
+    maker = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(maker)
+    if os.path.exists(maker.REGISTRY):
+        assert maker.resolve_with_reference_registry() == golden
+
+
 def test_benchmark_rows_record_format(tmp_path, monkeypatch):
     """The record written for the upstream benchmark runner: "[INFO] " + one JSON document with the
     runner's top-level keys, rows carrying every default field (benchmark/recording.py:37-53), non-finite
@@ -159,6 +182,11 @@ def test_benchmark_rows_record_format(tmp_path, monkeypatch):
     doc = json.loads(lines[0][len("[INFO] "):])
     assert doc["op_name"] == "sage_attention" and doc["result"][0]["latency_base"] is None
     assert set(R.ROW_DEFAULTS) <= set(doc["result"][0])
+    assert R.to_json_line({"a": [float("inf"), 1.5, {"b": float("-inf")}], "t": torch.float16}) == \
+        '{"a": [null, 1.5, {"b": null}], "t": "torch.float16"}'
+    x = torch.tensor([3.0, 4.0])
+    cos, rel = R.accuracy(x, torch.tensor([3.0, 0.0]))  # 3-4-5 triangle
+    assert abs(cos - 0.6) < 1e-6 and abs(rel - 4.0 / 3.0) < 1e-6
     assert R.baseline_name(torch.float16) == "torch_sdpa"
     assert R.baseline_name(torch.bfloat16) == "torch_sdpa_plus_bfloat16_cast"
     if not torch.cuda.is_available():
