@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsage_attention_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 SAGE_F16, SAGE_BF16, SAGE_F32 = 0, 1, 2
 MASK_NONE, MASK_BOOL, MASK_F32 = 0, 1, 2
@@ -30,6 +30,11 @@ class QuantParams(ctypes.Structure):
         ("blkq", c_i32), ("blkk", c_i32),
         ("q_mul", ctypes.c_float),
     ]
+
+
+class SmoothQuantParams(ctypes.Structure):
+    _fields_ = [("quant", QuantParams), ("km_out", ctypes.c_void_p), ("q_dot_km", ctypes.c_void_p),
+                ("workspace", ctypes.c_void_p)]
 
 
 class AttnParams(ctypes.Structure):
@@ -57,6 +62,7 @@ class FlashParams(ctypes.Structure):
 
 EXPORTS = (
     "sage_per_block_int8",
+    "sage_per_block_int8_smooth_k",
     "sage_attn_fwd",
     "sage_flash_attn_fwd",
     "sage_k_mean",
@@ -87,6 +93,8 @@ def load():
     lib.sage_hip_abi_version.restype = ctypes.c_int
     lib.sage_per_block_int8.argtypes = [ctypes.POINTER(QuantParams), ctypes.c_void_p]
     lib.sage_per_block_int8.restype = ctypes.c_int
+    lib.sage_per_block_int8_smooth_k.argtypes = [ctypes.POINTER(SmoothQuantParams), ctypes.c_void_p]
+    lib.sage_per_block_int8_smooth_k.restype = ctypes.c_int
     lib.sage_attn_fwd.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_void_p]
     lib.sage_attn_fwd.restype = ctypes.c_int
     lib.sage_flash_attn_fwd.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p]

@@ -25,7 +25,35 @@ using namespace sage;
 extern "C" const char* sage_hip_last_error(void) { return g_err; }
 extern "C" int sage_hip_abi_version(void) { return SAGE_HIP_ABI_VERSION; }
 
+static int check_quant_params(const sage_quant_params* p);
+
 extern "C" int sage_per_block_int8(const sage_quant_params* p, void* stream) {
+    if (int rc = check_quant_params(p)) return rc;
+    return launch_quant(*p, (hipStream_t)stream);
+}
+
+extern "C" int sage_per_block_int8_smooth_k(const sage_smooth_quant_params* sp, void* stream) {
+    if (!sp) return fail(SAGE_E_INVALID, "sage_per_block_int8_smooth_k: null params");
+    sage_quant_params p = sp->quant;
+    p.km.ptr = nullptr;  // the mean is computed here
+    if (int rc = check_quant_params(&p)) return rc;
+    if (!p.k.ptr || !sp->km_out || !sp->workspace)
+        return fail(SAGE_E_INVALID, "sage_per_block_int8_smooth_k: k, km_out and workspace are required");
+    if (p.batch <= 0 || p.heads_kv <= 0 || p.kv_len <= 0)
+        return fail(SAGE_E_INVALID, "sage_per_block_int8_smooth_k: batch, heads_kv and kv_len must be positive");
+    if (sp->q_dot_km) {
+        const int64_t d8 = p.head_dim / 8;
+        if (!p.q.ptr) return fail(SAGE_E_INVALID, "sage_per_block_int8_smooth_k: q_dot_km needs q");
+        if ((d8 & (d8 - 1)) != 0 || d8 > 64)
+            return fail(SAGE_E_UNSUPPORTED, "sage_per_block_int8_smooth_k: q_dot_km needs head_dim 8, 16, ..., 512");
+        if (p.heads_kv <= 0 || p.heads_q % p.heads_kv != 0)
+            return fail(SAGE_E_INVALID, "sage_per_block_int8_smooth_k: heads_q %lld is not a multiple of heads_kv %lld",
+                        (long long)p.heads_q, (long long)p.heads_kv);
+    }
+    return launch_smooth_quant(p, sp->km_out, sp->q_dot_km, sp->workspace, (hipStream_t)stream);
+}
+
+static int check_quant_params(const sage_quant_params* p) {
     if (!p) return fail(SAGE_E_INVALID, "sage_per_block_int8: null params");
     if (p->batch < 0 || p->heads_q < 0 || p->heads_kv < 0 || p->qo_len < 0 || p->kv_len < 0)
         return fail(SAGE_E_INVALID, "sage_per_block_int8: negative size");
@@ -47,7 +75,7 @@ extern "C" int sage_per_block_int8(const sage_quant_params* p, void* stream) {
         if (p->in_dtype == SAGE_F32 && p->diff_dtype != SAGE_F32)
             return fail(SAGE_E_INVALID, "sage_per_block_int8: fp32 K needs diff_dtype fp32");
     }
-    return launch_quant(*p, (hipStream_t)stream);
+    return SAGE_OK;
 }
 
 extern "C" int64_t sage_k_mean_workspace_bytes(int64_t batch, int64_t heads_kv, int64_t kv_len, int64_t head_dim) {

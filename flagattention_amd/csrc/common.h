@@ -22,6 +22,7 @@ inline int dtype_bytes(int dt) { return dt == SAGE_F32 ? 4 : 2; }
 int launch_quant(const sage_quant_params& p, hipStream_t stream);
 int launch_kmean(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype, int64_t B, int64_t H, int64_t N,
                  int64_t D, void* workspace, hipStream_t stream);
+int launch_smooth_quant(const sage_quant_params& p, void* km_out, float* q_dot_km, void* workspace, hipStream_t stream);
 // Device address of the library's static scratch array on the current device (SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES).
 int static_scratch(void** out);
 int launch_attn(const sage_attn_params& p, hipStream_t stream);

@@ -5,9 +5,9 @@ alias of ``forward``).  ``sageattn`` is the one-call convenience every caller of
 functions writes by hand (README.md:259-275 of the reference).
 """
 from .attention import forward
-from .quant import k_mean, per_block_int8
+from .quant import k_mean, per_block_int8, per_block_int8_smooth_k
 from .api import sageattn
 
 sage_attention = forward
 
-__all__ = ["sage_attention", "forward", "per_block_int8", "k_mean", "sageattn"]
+__all__ = ["sage_attention", "forward", "per_block_int8", "per_block_int8_smooth_k", "k_mean", "sageattn"]

@@ -6,7 +6,7 @@ import math
 import torch
 
 from .attention import forward
-from .quant import k_mean, per_block_int8
+from .quant import per_block_int8, per_block_int8_smooth_k
 
 
 def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True,
@@ -22,18 +22,17 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
         output_dtype = q.dtype
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
-    km = k_mean(k, tensor_layout) if smooth_k else None
-    q8, qs, k8, ks = per_block_int8(q, k, km=km, sm_scale=sm_scale, tensor_layout=tensor_layout)
+    q_dot_km = None
+    if smooth_k:
+        q8, qs, k8, ks, _, q_dot_km = per_block_int8_smooth_k(q, k, sm_scale=sm_scale, tensor_layout=tensor_layout,
+                                                             with_q_dot_km=return_lse)
+    else:
+        q8, qs, k8, ks = per_block_int8(q, k, sm_scale=sm_scale, tensor_layout=tensor_layout)
     o, lse2 = forward(q8, k8, v, qs, ks, tensor_layout=tensor_layout, output_dtype=output_dtype,
                       return_lse=return_lse, causal=is_causal)
     if not return_lse:
         return o
     lse = lse2 * math.log(2.0)
-    if km is not None:
-        hnd = tensor_layout == "HND"
-        qh = q if hnd else q.transpose(1, 2)
-        kmh = km if hnd else km.transpose(1, 2)
-        groups = qh.shape[1] // kmh.shape[1]
-        kmh = kmh.repeat_interleave(groups, dim=1) if groups > 1 else kmh
-        lse = lse + sm_scale * (qh.float() * kmh.float()).sum(dim=-1)
+    if q_dot_km is not None:
+        lse = torch.addcmul(lse, q_dot_km, torch.tensor(sm_scale, dtype=torch.float32, device=lse.device))
     return o, lse

@@ -69,9 +69,21 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
     (default ``head_dim ** -0.5``) before quantization, K by nothing; ``km`` (any tensor
     broadcastable to ``k``) is subtracted from K first with torch's rounding.
 
-    ``smooth_k=True`` (keyword only, not in the reference) computes ``km = k_mean(k)`` when no
-    ``km`` is given.
+    ``smooth_k=True`` (keyword only, not in the reference) uses ``km = k_mean(k)`` when no
+    ``km`` is given, computed inside the same library call.
     """
+    return _quantize(q, k, km, BLKQ, BLKK, sm_scale, tensor_layout, smooth_k and km is None, False)[:4]
+
+
+def per_block_int8_smooth_k(q, k, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", with_q_dot_km=False):
+    """``per_block_int8(q, k, km=k_mean(k))`` in one library call.  Returns ``(q_int8, q_scale, k_int8, k_scale,
+    km, q_dot_km)``: ``km`` as ``k_mean`` returns it, ``q_dot_km`` (``[B, Hq, M]`` fp32, or None unless asked for)
+    the dot product of every query row with the mean of its KV head: smoothing lowers every logit ``q.k`` of
+    the row by that amount."""
+    return _quantize(q, k, None, BLKQ, BLKK, sm_scale, tensor_layout, True, with_q_dot_km)
+
+
+def _quantize(q, k, km, BLKQ, BLKK, sm_scale, tensor_layout, smooth, want_dot):
     if tensor_layout not in ("HND", "NHD"):
         raise ValueError(f"Unknown tensor layout: {tensor_layout}")
     hnd = tensor_layout == "HND"
@@ -87,15 +99,19 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
         raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
     if k.device != q.device:
         raise ValueError("q and k must be on the same device")
-    if km is None and smooth_k:
-        km = k_mean(k, tensor_layout)
     if sm_scale is None:
         sm_scale = head_dim ** -0.5
     BLKQ, BLKK = int(BLKQ), int(BLKK)
     if BLKQ <= 0 or BLKK <= 0:
         raise ValueError("BLKQ and BLKK must be positive")
+    # one library call does mean + smoothing + quantization when Q and K share a dtype and there is a K to average
+    fused = smooth and q.dtype == k.dtype and b > 0 and h_kv > 0 and kv_len > 0 and \
+        (not want_dot or (h_qo % h_kv == 0 and head_dim in (8, 16, 32, 64, 128, 256, 512)))
+    if smooth and not fused:
+        km = k_mean(k, tensor_layout)
 
     lib = _lib.load()
+    dot = None
     with torch.cuda.device(q.device):
         q_int8 = torch.empty(q.shape, dtype=torch.int8, device=q.device)
         k_int8 = torch.empty(k.shape, dtype=torch.int8, device=k.device)
@@ -112,6 +128,23 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
         p.k_int8 = tensor_desc(k_int8, hnd)
         p.km = _lib.SageTensor(None, 0, 0, 0)
         p.km_dtype = p.diff_dtype = _lib.SAGE_F32
+        stream = current_stream_ptr(q.device)
+        if fused:
+            sp = _lib.SmoothQuantParams()
+            p.in_dtype = DTYPE_CODE[q.dtype]
+            p.q = tensor_desc(q, hnd)
+            p.k = tensor_desc(k, hnd)
+            sp.quant = p
+            km_flat = torch.empty((b, h_kv, head_dim), dtype=k.dtype, device=k.device)
+            ws = torch.empty(max(1, lib.sage_k_mean_workspace_bytes(b, h_kv, kv_len, head_dim) // 4),
+                             dtype=torch.float32, device=k.device)
+            sp.km_out, sp.workspace = km_flat.data_ptr(), ws.data_ptr()
+            if want_dot:
+                dot = torch.empty((b, h_qo, qo_len), dtype=torch.float32, device=q.device)
+                sp.q_dot_km = dot.data_ptr()
+            _lib.check(lib.sage_per_block_int8_smooth_k(ctypes.byref(sp), stream), "sage_per_block_int8_smooth_k")
+            km = km_flat.view(b, h_kv, 1, head_dim) if hnd else km_flat.view(b, 1, h_kv, head_dim)
+            return q_int8, q_scale, k_int8, k_scale, km, dot
         km_keepalive = None
         if km is not None:
             require_gpu(km, "km")
@@ -124,7 +157,6 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
             p.km = tensor_desc(kme, hnd)
             p.km_dtype = DTYPE_CODE[km.dtype]
             p.diff_dtype = DTYPE_CODE[torch.result_type(k, km)]
-        stream = current_stream_ptr(q.device)
         if q.dtype == k.dtype:
             p.in_dtype = DTYPE_CODE[q.dtype]
             p.q = tensor_desc(q, hnd)
@@ -137,4 +169,9 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
             p.in_dtype, p.q, p.k = DTYPE_CODE[k.dtype], null, tensor_desc(k, hnd)
             _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
         del km_keepalive
-    return q_int8, q_scale, k_int8, k_scale
+    if want_dot and km is not None:  # (mixed dtypes or an unusual head_dim: the dot product is taken by torch)
+        qh, kmh = (q, km) if hnd else (q.transpose(1, 2), km.transpose(1, 2))
+        groups = h_qo // h_kv
+        kmh = kmh.repeat_interleave(groups, dim=1) if groups > 1 else kmh
+        dot = (qh.float() * kmh.float()).sum(dim=-1)
+    return q_int8, q_scale, k_int8, k_scale, km, dot

@@ -106,6 +106,30 @@ int sage_k_mean(const sage_tensor* k, int32_t k_dtype, void* km_out, int32_t out
                 int64_t heads_kv, int64_t kv_len, int64_t head_dim, void* workspace, void* stream);
 
 /*
+ * per_block_int8 with the K smoothing done by the library: km = sage_k_mean(k), then the quantization of
+ * `k - km` and of q, as three launches instead of five (the Q blocks run side by side with the first pass over
+ * K).  The reference leaves km to its caller (quant_per_block.py:49,53-54); its README's call sequence
+ * (README.md:259-275: mean, per_block_int8, forward) is what this entry point stands for.  Results are
+ * bit-identical to sage_k_mean followed by sage_per_block_int8 with that km.
+ *
+ *   quant        as for sage_per_block_int8; q and k share in_dtype; km / km_dtype / diff_dtype are ignored
+ *                (the mean has k's dtype, so the difference is rounded to k's dtype); q.ptr may be NULL
+ *   km_out       [B, Hkv, D] contiguous, in_dtype: the mean that was subtracted (required)
+ *   q_dot_km     optional [B, Hq, M] fp32: sum over head_dim of fp32(q) * fp32(km of the row's KV head) — the
+ *                amount by which smoothing lowers every logit q.k of that row before sm_scale, which a caller
+ *                adds back to a log-sum-exp of the smoothed scores; NULL = not wanted
+ *   workspace    sage_k_mean_workspace_bytes(batch, heads_kv, kv_len, head_dim) bytes, 16-byte aligned
+ */
+typedef struct sage_smooth_quant_params {
+    sage_quant_params quant;
+    void* km_out;
+    float* q_dot_km;
+    void* workspace;
+} sage_smooth_quant_params;
+
+int sage_per_block_int8_smooth_k(const sage_smooth_quant_params* p, void* stream);
+
+/*
  * sage_k_mean without a workspace argument and without any allocation: no counterpart in the reference.
  * It is for callers that cannot allocate device memory around the call (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): the chunk partials go to a fixed array inside the
@@ -150,7 +174,7 @@ const char* sage_hip_last_error(void);
 
 /* ABI version of this header; bumped when a struct layout changes. */
 int sage_hip_abi_version(void);
-#define SAGE_HIP_ABI_VERSION 2
+#define SAGE_HIP_ABI_VERSION 3
 
 #ifdef __cplusplus
 }

@@ -300,20 +300,35 @@ def test_seeded_shape_sweep(case, gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
 
 
-def test_sageattn_wrapper_lse(gpu_device):
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("smooth_k", [False, True])
+@pytest.mark.parametrize("d,dtype,hq,hkv", [(128, torch.bfloat16, 4, 2), (64, torch.float16, 3, 3)])
+def test_sageattn_wrapper_lse(layout, causal, smooth_k, d, dtype, hq, hkv, gpu_device):
+    """The one-call wrapper in every branch (both layouts, causal flag, with and without K smoothing, grouped
+    heads) against fp32 attention of the unquantized inputs; the log-sum-exp is the one of the UNSMOOTHED
+    logits sm_scale * q . k (natural log), whatever smoothing did to the scores inside."""
     from flag_attn.sage_attention import sageattn
 
+    m, n = 300, 500
     g = torch.Generator().manual_seed(4)
-    q = torch.randn(1, 4, 300, 128, generator=g).to(torch.bfloat16).to(gpu_device)
-    k = (torch.randn(1, 2, 500, 128, generator=g) + 1.5).to(torch.bfloat16).to(gpu_device)
-    v = torch.randn(1, 2, 500, 128, generator=g).to(torch.bfloat16).to(gpu_device)
-    o, lse = sageattn(q, k, v, return_lse=True)
-    kk, vv = k.repeat_interleave(2, 1).float(), v.repeat_interleave(2, 1).float()
-    s = (q.float() @ kk.transpose(-1, -2)) * 128 ** -0.5
-    ref = torch.softmax(s, -1) @ vv
-    cos, rel, _ = O.accuracy_metrics(o.cpu(), ref.cpu())
+    q = torch.randn(1, hq, m, d, generator=g).to(dtype)
+    k = (torch.randn(1, hkv, n, d, generator=g) + 1.5 * torch.randn(1, hkv, 1, d, generator=g)).to(dtype)
+    v = torch.randn(1, hkv, n, d, generator=g).to(dtype)
+    kk, vv = k.repeat_interleave(hq // hkv, 1).float(), v.repeat_interleave(hq // hkv, 1).float()
+    s = (q.float() @ kk.transpose(-1, -2)) * d ** -0.5
+    if causal:
+        s = s.masked_fill(~O.causal_mask(m, n), float("-inf"))
+    ref, ref_lse = torch.softmax(s, -1) @ vv, torch.logsumexp(s, -1)
+    args = [t.to(gpu_device) if layout == "HND" else t.transpose(1, 2).contiguous().to(gpu_device) for t in (q, k, v)]
+    o, lse = sageattn(*args, tensor_layout=layout, is_causal=causal, smooth_k=smooth_k, return_lse=True)
+    assert o.dtype == dtype and o.shape == args[0].shape and lse.shape == (1, hq, m)
+    o_only = sageattn(*args, tensor_layout=layout, is_causal=causal, smooth_k=smooth_k)
+    assert torch.equal(o_only, o)
+    oh = o if layout == "HND" else o.transpose(1, 2)
+    cos, rel, _ = O.accuracy_metrics(oh.cpu(), ref)
     assert cos >= 0.999 and rel <= 0.05
-    torch.testing.assert_close(lse, torch.logsumexp(s, -1), atol=5e-2, rtol=1e-3)
+    torch.testing.assert_close(lse.cpu(), ref_lse, atol=5e-2, rtol=1e-3)
 
 
 def test_side_stream_and_graph_replay(gpu_device):

@@ -47,6 +47,7 @@ def test_struct_layouts_match_header():
     fields = {
         "sage_quant_params": (_lib.QuantParams, ["q", "k", "km", "q_int8", "k_int8", "q_scale", "k_scale", "batch",
                                                  "head_dim", "in_dtype", "km_dtype", "diff_dtype", "blkq", "blkk", "q_mul"]),
+        "sage_smooth_quant_params": (_lib.SmoothQuantParams, ["quant", "km_out", "q_dot_km", "workspace"]),
         "sage_attn_params": (_lib.AttnParams, ["q", "out", "q_scale", "k_scale", "lse", "mask", "mask_stride_b",
                                                "mask_stride_n", "batch", "head_dim", "v_dtype", "out_dtype", "mask_kind", "causal"]),
         "sage_flash_params": (_lib.FlashParams, ["q", "out", "log_normalizer", "batch", "head_dim", "dtype", "out_dtype",

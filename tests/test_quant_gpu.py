@@ -218,3 +218,37 @@ def test_seeded_quantizer_sweep(case, gpu_device):
     want = O.per_block_int8(q, k, km=km, **kw)
     got = per_block_int8(q.to(gpu_device), k.to(gpu_device), km=_gpu(km, gpu_device), **kw)
     _assert_bit_exact(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("shape", [(2, 4, 2, 384, 512, 128), (1, 6, 3, 300, 449, 64), (2, 2, 2, 128, 64, 128), (1, 3, 1, 77, 1000, 32),
+                                   (1, 2, 2, 256, 192, 96)])
+def test_smoothing_inside_the_library_call(dtype, layout, shape, gpu_device):
+    """per_block_int8_smooth_k (mean, smoothing and quantization in one call, Q blocks side by side with the
+    first pass over K) against the oracle, bit for bit, with and without the q . km output; whole blocks,
+    tails, grouped heads, head dims that take the fused first launch (64, 128) and ones that do not."""
+    from flag_attn.sage_attention import k_mean, per_block_int8, per_block_int8_smooth_k
+
+    b, hq, hkv, m, n, d = shape
+    g = torch.Generator().manual_seed(1234)
+    q = torch.randn(b, hq, m, d, generator=g).to(dtype)
+    k = (torch.randn(b, hkv, n, d, generator=g) + 2.0 * torch.randn(1, hkv, 1, d, generator=g)).to(dtype)
+    if layout == "NHD":
+        q, k = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+    km = C.k_mean_fixed_order(k, layout)
+    want = C.per_block_int8(q, k, km=km, tensor_layout=layout)
+    qd, kd = q.to(gpu_device), k.to(gpu_device)
+    qh, kmh = (q, km) if layout == "HND" else (q.transpose(1, 2), km.transpose(1, 2))
+    dot_want = (qh.double() * kmh.repeat_interleave(hq // hkv, dim=1).double()).sum(-1)
+    for with_dot in (False, True):
+        got = per_block_int8_smooth_k(qd, kd, tensor_layout=layout, with_q_dot_km=with_dot)
+        _assert_bit_exact(got[:4], want)
+        assert got[4].shape == km.shape and torch.equal(got[4].cpu().view(torch.uint8), km.contiguous().view(torch.uint8))
+        if with_dot:
+            assert got[5].shape == (b, hq, m) and got[5].dtype == torch.float32
+            torch.testing.assert_close(got[5].cpu().double(), dot_want, rtol=2e-5, atol=2e-4)
+        else:
+            assert got[5] is None
+    _assert_bit_exact(per_block_int8(qd, kd, tensor_layout=layout, smooth_k=True), want)
+    assert torch.equal(k_mean(kd, layout).cpu().view(torch.uint8), km.contiguous().view(torch.uint8))
