@@ -166,9 +166,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // the direct-to-LDS loads are tracked with
     typedef __attribute__((address_space(4))) const float* const_f32_ptr;
     const const_f32_ptr ksp = (const_f32_ptr)(uintptr_t)(a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk);
-    auto step_scale = [&](int j) {  // scale of the scores of step j
+    auto step_scale = [&](int j, bool hides) {  // scale of the scores of step j (hides: the step may hold hidden keys)
         float s = INT8 ? qs * ksp[j] : qs;
-        if (CAUSAL) s = fmaxf(s, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
+        if (CAUSAL && hides) s = fmaxf(s, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
         return s;
     };
     const int8_t* kg = a.k + ((int64_t)b * a.ks_b + (int64_t)hk * a.ks_h) * QB;
@@ -220,15 +220,16 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     }
     // unit e < NK of a wave's share of one K tile + one V tile: a K instruction; the rest: V instructions.
     // kt / vt: index of the tile behind ktile / vtile
-    auto dma_unit = [&](auto ec, int kbuf, const unsigned char* ktile, int kt, int vbuf, const unsigned char* vtile, int vt) {
+    auto dma_unit = [&](auto ec, auto hc, int kbuf, const unsigned char* ktile, int kt, int vbuf, const unsigned char* vtile, int vt) {
         constexpr int e = decltype(ec)::value;
+        constexpr bool HIDES = decltype(hc)::value;  // false: the caller knows that neither tile is a ragged last one
         if constexpr (e < F::NK) {
-            const bool cut = ragged && kt == a.nk - 1;
+            const bool cut = HIDES && ragged && kt == a.nk - 1;
             dma16(cut ? ktile : ktile + e * k_instr_bytes, cut ? k_goff_last[e] : k_goff,
                   lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
         } else {
             constexpr int ev = e - F::NK;
-            const bool cut = ragged && vt == a.nk - 1;
+            const bool cut = HIDES && ragged && vt == a.nk - 1;
             dma16(cut ? vtile : vtile + ev * v_instr_bytes, cut ? v_goff_last[ev] : v_goff,
                   lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
@@ -352,18 +353,18 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg);
     const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg);
     int k_tile = 0, v_tile = 0;  // indices of the tiles behind k_fetch / v_fetch
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<1>{}, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
     if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
+    sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<1>{}, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
     if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
-    sfor<F::NK>([&](auto ec) { dma_unit(ec, 2, k_fetch, k_tile, 2, v_fetch, v_tile); });
+    sfor<F::NK>([&](auto ec) { dma_unit(ec, IC<1>{}, 2, k_fetch, k_tile, 2, v_fetch, v_tile); });
     // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
     if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);
     sbuf[0][1] = qk_tile(smem, 1);
-    sc = step_scale(0);
+    sc = step_scale(0, true);
     {   // the row maximum of the first tile is the reference point the row starts from
         float raw_max = -INFINITY;
         const bool masked0 = CAUSAL && (BN - 1 > wlim);
@@ -378,8 +379,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // instructions); the two waves that share a SIMD run half a step
     // apart (see the barrier before the loop), so one feeds the matrix core while the other
     // occupies the VALU.  Two barriers per step.
-    auto body = [&](auto pc, int step) {
+    // HIDES = false is the body for steps that hide no key of this step or the next and fetch no ragged tile:
+    // the code of the instance that cannot hide keys at all.  Both bodies pass the same two barriers, so the
+    // waves of a workgroup may be in different ones.
+    auto body = [&](auto pc, auto hc, int step) {
         constexpr int P = decltype(pc)::value;  // == step & 1
+        constexpr bool HIDES = CAUSAL && decltype(hc)::value;
         // tile t of K (of V) lives in LDS buffer t % 4: this step reads K of step+1 and V of step, and
         // fetches K of step+3 and V of step+2 into the buffers that K of step-1 and V of step-2 left
         int kaddr[F::KSTEPS], vaddr[F::DTILES];
@@ -429,7 +434,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
         // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
         // instruction.
-        sfor<NDMA>([&](auto ec) { dma_unit(ec, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
+        sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
         vec16 pf[4];
         float lsum = 0.0f;
         const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
@@ -502,7 +507,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             }
         };
         if constexpr (kSumsEarly) large = __builtin_amdgcn_ballot_w64(!(lsum < kSumLimit));
-        sc = step_scale(min(step + 1, nsteps - 1));
+        sc = step_scale(min(step + 1, nsteps - 1), HIDES);
         __builtin_amdgcn_sched_barrier(0);
         // The first K fragments of the coming MFMA phase are requested before the barrier (their tile
         // landed a step ago), so the phase does not open with an LDS round trip.
@@ -516,7 +521,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 
         // ===== MFMA phase =====
         __builtin_amdgcn_s_setprio(1);
-        const bool masked_n = CAUSAL && (n0 + 2 * BN - 1 > wlim);
+        const bool masked_n = HIDES && (n0 + 2 * BN - 1 > wlim);
         sfor<NSLOTS>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if constexpr (i < QK_SLOTS) {
@@ -563,7 +568,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                 if constexpr (j + VDIST < PV_SLOTS) read_v(IC<j + VDIST>{});
                 // hidden keys of the next step's scores (Q.K^T finished above) are set to -inf under the
                 // P.V instructions
-                if constexpr (CAUSAL) {
+                if constexpr (HIDES) {
                     sfor<8 / PV_SLOTS + (8 % PV_SLOTS != 0)>([&](auto rc) {
                         constexpr int u = j * (8 / PV_SLOTS + (8 % PV_SLOTS != 0)) + decltype(rc)::value;
                         if constexpr (u < 8) {
@@ -594,9 +599,24 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     if (wave >= kFastWaves / 2) __syncthreads();  // second half of the waves runs one phase behind
     // The loop always runs an even number of steps (no exit between the two parities: the accumulators
     // then stay in one set of registers); after an odd nsteps the extra step multiplies V by P = 0.
-    for (int step = 0; step < nsteps; step += 2) {
-        body(IC<0>{}, step);
-        body(IC<1>{}, step + 1);
+    // Steps before `hide_from` (even) take the lean body: step s hides keys when its tile reaches past the limit
+    // of the wave's first row, which the body of step s - 1 prepares; a ragged last tile is fetched three (K) or
+    // two (V) steps ahead.
+    int hide_from = 0;
+    if (CAUSAL) {
+        const int first_hidden_step = (__builtin_amdgcn_readfirstlane(wlim) + 1) / BN;  // tile that holds key wlim + 1 (may lie past the last step); wave-uniform
+        hide_from = max(min(first_hidden_step - 1, ragged ? a.nk - 4 : nsteps), 0) & ~1;
+    }
+    int step = 0;
+    if (CAUSAL) {
+        for (; step < min(hide_from, nsteps); step += 2) {
+            body(IC<0>{}, IC<0>{}, step);
+            body(IC<1>{}, IC<0>{}, step + 1);
+        }
+    }
+    for (; step < nsteps; step += 2) {
+        body(IC<0>{}, IC<1>{}, step);
+        body(IC<1>{}, IC<1>{}, step + 1);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // every direct-to-LDS load of this wave has landed
     if (wave < kFastWaves / 2) __syncthreads();
