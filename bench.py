@@ -34,10 +34,23 @@ PEAK_INT8_TOPS = 5000.0
 PEAK_16BIT_TFLOPS = 2500.0
 PEAK_MIXED_TOPS = 1.0 / (0.5 / PEAK_INT8_TOPS + 0.5 / PEAK_16BIT_TFLOPS)  # 3333.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per attention launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
-# dispatch, scaled by the factors a 256 MiB read+write kernel gives in the same run: 2.00 / 1.00);
-# summaries under profiles/.  None = not measured for that workload.
-MEASURED_ATTN_TRAFFIC_BYTES = {"c2": 402.9e6}
+# HBM bytes per attention launch come from profiles/attention_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch) scaled by what the same counters read for a copy of known size in the same run.  One line
+# per workload: "<name> <bytes per launch> ...".  A workload without a line reports traffic null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attention_hbm_traffic.txt")
+
+
+def measured_traffic_bytes(name, op="sage_attention"):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) >= 3 and parts[0] == op and parts[1] == name:
+                    return float(parts[2])
+    except OSError:
+        pass
+    return None
+
 
 WORKLOADS = {
     # name: (B, H, N, D, dtype, layout, causal, description)
@@ -167,7 +180,7 @@ def main_flash(args):
         "parity": parity,
         "roofline": {"kernel": "sage_attn_fwd_fast_kernel (16-bit Q, K instance)", "bound": "mfma",
                      "achieved": round(ops / (avg * 1e-3) / 1e12, 2), "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": None,
+                     "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": measured_traffic_bytes(name, "flash_attention"),
                      "algorithmic_bytes_per_launch": 4 * numel * 2, "algorithmic_ops_per_launch": ops,
                      "avg_launch_ms": round(avg, 4)},
     }
@@ -244,23 +257,33 @@ def main():
     # ---- timed region: W warm-up steps, then exactly K steps.  The GPU clock needs about 0.1 s of load to
     #      leave its idle state (the first launches after an idle gap run 10-25 % slower), so the warm-up
     #      is never shorter than that, whatever W says; the timed region is exactly K steps.
+    def timed(nsteps):
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(nsteps)]
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        for i in range(nsteps):
+            step(evs[i])
+        torch.cuda.synchronize()
+        return time.perf_counter() - t_start, evs
+
+    time.sleep(1.0)  # the checks above kept the GPU busy: let it fall idle, as a fresh caller would find it
     t_ramp = time.perf_counter()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # (a) exactly what was asked for: W warm-up steps from idle, then K steps (the clock may still be ramping)
+    wall_asked, ev_asked = timed(args.steps)
+    # (b) the sustained rate, reported as `value`: the warm-up is stretched to at least 0.15 s of load
     ramp_steps = 0
     while time.perf_counter() - t_ramp < 0.15:
         for _ in range(10):
             step()
         torch.cuda.synchronize()
         ramp_steps += 10
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(events[i])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall, events = timed(args.steps)
+    # (c) cold: one step after a second of idleness, no warm-up at all
+    time.sleep(1.0)
+    wall_cold, ev_cold = timed(1)
     quant_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
     attn_ms = [e[1].elapsed_time(e[2]) for e in events]
     attn_avg = sum(attn_ms) / len(attn_ms)
@@ -268,19 +291,26 @@ def main():
     quant_med = quant_ms[len(quant_ms) // 2]
     ms_per_step = wall / args.steps * 1e3
 
-    ops = algorithmic_ops(name)
+    ops = ops_of_step = algorithmic_ops(name)
     esz = 2
     numel = b * h * n * d
     quant_bytes = (esz + 1) * 2 * numel + (esz * numel if smooth else 0)  # Q,K read+write (+ K read by the mean)
     value = ops / (ms_per_step * 1e-3) / 1e12
     attn_tops = ops / (attn_avg * 1e-3) / 1e12
     result = {
-        "metric": "effective TOPS + % of dense MFMA peak, B4 H32 N4096 D128 bf16; us/call",
+        "metric": f"effective TOPS + % of dense MFMA peak, B{b} H{h} N{n} D{d} {'bf16' if dtype == torch.bfloat16 else 'fp16'}; us/call",
         "value": round(value, 2),
-        "unit": "TOPS (effective: 4*B*H*N^2*D ops per call / time of k_mean + per_block_int8 + forward)",
+        "unit": "TOPS (effective: 4*B*H*N^2*D ops per call (causal: visible pairs only) / time of K mean + per_block_int8 + forward)",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup, "clock_ramp_steps": ramp_steps,
+        "timing_note": "value / ms_per_step: K steps at the sustained clock (warm-up stretched to >= 0.15 s of load); "
+                       "as_requested: K steps right after the W warm-up steps asked for, from an idle GPU; cold: one step after 1 s idle",
+        "as_requested": {"ms_per_step": round(wall_asked / args.steps * 1e3, 4),
+                         "value": round(ops_of_step / (wall_asked / args.steps) / 1e12, 2),
+                         "attention_us_avg": round(sum(e[1].elapsed_time(e[2]) for e in ev_asked) / len(ev_asked) * 1e3, 1)},
+        "cold": {"ms_per_step": round(wall_cold * 1e3, 4), "value": round(ops_of_step / wall_cold / 1e12, 2),
+                 "attention_us": round(ev_cold[0][1].elapsed_time(ev_cold[0][2]) * 1e3, 1)},
         "ms_per_step": round(ms_per_step, 4),
         "us_per_call": round(ms_per_step * 1e3, 1),
         "higher_is_better": True,
@@ -302,7 +332,8 @@ def main():
         },
         "quant": {"us_per_call_median": round(quant_med * 1e3, 1),
                   "gbps": round(quant_bytes / (quant_med * 1e-3) / 1e9, 1),
-                  "scope": "k_mean (2 launches) + per_block_int8 (2 launches)" if smooth else "per_block_int8 (2 launches)"},
+                  "scope": "per_block_int8 with the K mean inside (3 launches: Q blocks + K chunk sums, mean, K blocks)" if smooth
+                  else "per_block_int8 (2 launches)"},
         "parity": {"int8_bit_exact": int8_exact, "scale_bit_exact": scale_exact, "cosine": cos, "max_abs_err": max_abs,
                    "checked_on": "batch 0, heads 0-1 (quantizer) / head 0 (attention) of this workload vs the CPU oracle"},
         "roofline": {
@@ -312,8 +343,8 @@ def main():
             "peak": round(PEAK_MIXED_TOPS, 1),
             "unit": "TFLOP/s",
             "frac": round(attn_tops / PEAK_MIXED_TOPS, 4),
-            "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get(name),
-            "traffic_unit": "bytes per launch (offline rocprofv3 counters, see profiles/)",
+            "traffic": measured_traffic_bytes(name),
+            "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, read from profiles/attention_hbm_traffic.txt)",
             "algorithmic_bytes_per_launch": numel * (1 + 1 + esz) + numel * out_dtype.itemsize,
             "peak_note": "mixed dense-MFMA roofline: half the ops INT8 at 5000 TOP/s, half 16-bit at 2500 TFLOP/s",
             "algorithmic_ops_per_launch": ops,

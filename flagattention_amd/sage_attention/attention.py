@@ -53,8 +53,16 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
         raise ValueError(f"v {tuple(v.shape)} must have k's shape {tuple(k.shape)}")
     if k.shape[0] != b or k.shape[-1] != head_dim:
         raise ValueError(f"q {tuple(q.shape)} and k {tuple(k.shape)} disagree on batch or head_dim")
+    if head_dim in (16, 32):
+        # Zero channels change neither Q.K^T nor the first head_dim columns of P.V: run at head_dim 64 on padded
+        # copies (the reference takes whatever its compiler's dot takes, attn_qk_int8_per_block.py:161,185).
+        pad = (0, 64 - head_dim)
+        qp, kp, vp = (torch.nn.functional.pad(t, pad) for t in (q, k, v))
+        o, lse = forward(qp, kp, vp, q_scale, k_scale, tensor_layout, attn_mask, output_dtype, return_lse, maxnreg,
+                         causal=causal)
+        return o[..., :head_dim].contiguous(), lse
     if head_dim not in (64, 128):
-        raise ValueError(f"head_dim {head_dim} not supported (64 or 128)")
+        raise ValueError(f"head_dim {head_dim} not supported (16, 32, 64 or 128)")
     if h_kv == 0 or h_qo % h_kv != 0:
         raise ValueError(f"num_qo_heads {h_qo} must be a multiple of num_kv_heads {h_kv}")
     nq = (qo_len + BLOCK_M - 1) // BLOCK_M

@@ -300,6 +300,31 @@ def test_seeded_shape_sweep(case, gpu_device):
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("d", [16, 32])
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+def test_small_head_dims_run_padded(d, layout, gpu_device):
+    """head_dim 16 and 32 (the quantizer takes them natively; the attention wrapper pads to 64)."""
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(2, 4, 200, d, generator=g).to(torch.float16)
+    k = torch.randn(2, 2, 333, d, generator=g).to(torch.float16)
+    v = torch.randn(2, 2, 333, d, generator=g).to(torch.float16)
+    if layout == "NHD":
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    want = O.per_block_int8(q, k, tensor_layout=layout)
+    got = sa.per_block_int8(q.to(gpu_device), k.to(gpu_device), tensor_layout=layout)
+    for a, b in zip(got, want):
+        assert torch.equal(a.cpu(), b)
+    for causal in (False, True):
+        o, lse = sa.sage_attention(got[0], got[2], v.to(gpu_device), got[1], got[3], tensor_layout=layout, causal=causal,
+                                   return_lse=True)
+        exp, exp_lse = O.attention_dequant(want[0], want[2], v, want[1], want[3], layout, causal=causal)
+        assert o.shape == q.shape and o.is_contiguous()
+        _gate(o, exp)
+        torch.testing.assert_close(lse.cpu(), exp_lse, atol=6e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("layout", ["HND", "NHD"])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("smooth_k", [False, True])
