@@ -80,6 +80,10 @@ template <> struct PV<_Float16> {
 // head_dim 64 / 128, V dtype fp16 / bf16.
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream);
 
+// The same kernel under a bool mask tensor, where fast_serves_mask() says so (a.mask set, MODE_MASK_BOOL).
+bool fast_serves_mask(const AttnArgs& a);
+int launch_fast_masked(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream);
+
 // The same kernel on 16-bit Q and K (dense attention); causal with any qo_len / kv_len.
 int launch_flash(const AttnArgs& a, int head_dim, int dtype, bool causal, hipStream_t stream);
 

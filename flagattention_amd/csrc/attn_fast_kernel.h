@@ -101,14 +101,28 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 // QB = 1: int8 Q and K with per-block scales (SageAttention).  QB = 2: Q and K in V's 16-bit type, one
 // scale for the whole call (dense attention); in bytes a 16-bit K row of head_dim D is laid out, loaded
 // and read exactly like an int8 row of head_dim 2 D.
-template <int D, typename VT, bool CAUSAL, int QB>
+// MASK: a bool mask tensor [B, Hq, M, N] (bytes 0 / 1, rows 16-byte aligned, kv_len a multiple of 16) on top of
+// the key-hiding instance.  Every wave stages the 32 x 64 mask bytes of its own rows and step in a private slice
+// of LDS (direct-to-LDS loads, three steps resident) and multiplies P by them.  The reference's arithmetic for
+// rows that have not seen a visible key yet (scores of hidden keys are s - 1e6, not -inf:
+// attn_qk_int8_per_block.py:46-52) and its skipping of 128 x 64 tiles without a visible key (:33-36) are
+// served by the path that redoes a step: such rows start from the reference point -inf, which drives every
+// step into that path until the row has seen a key.  Additive masks and masks with unaligned rows stay with the
+// general kernel (attn_fwd.hip).
+constexpr int kMaskSlots = 3;                       // steps of mask bytes resident per wave
+constexpr int kMaskWaveBytes = 32 * BN;            // 32 rows x 64 keys x 1 byte
+constexpr int kMaskBytes = kMaskSlots * kFastWaves * kMaskWaveBytes;
+constexpr float kMaskedScore = -1.0e6f;            // what the reference adds to the score of a hidden key
+
+template <int D, typename VT, bool CAUSAL, int QB, bool MASK = false>
 __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
     using F = FT<D, QB>;
     constexpr bool INT8 = QB == 1;
+    static_assert(!MASK || (CAUSAL && INT8), "the mask instance builds on the key-hiding int8 instance");
     constexpr float BIAS = INT8 ? kBias : 0.0f;  // what the bits of a fresh score accumulator read as a float
     using PVT = PV<VT>;
     using vec16 = typename PVT::vec;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL];
+    __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL + (MASK ? kMaskBytes : 0)];
 
 
     // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
@@ -234,8 +248,61 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                   lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
     };
-    constexpr int NDMA = F::NK + F::NV;  // loads per wave per step
+    constexpr int NDMA = F::NK + F::NV + (MASK ? 2 : 0);  // loads per wave per step
+    constexpr int NDMA_KV = F::NK + F::NV;
 
+    // ---- mask staging (MASK): the wave's 32 rows x 64 keys of step t go to slot t % 3 of its own 2 KB slices, row
+    //      after row (instruction e carries rows 16 e .. 16 e + 15, four lanes per row, so that neighbouring lanes
+    //      read neighbouring bytes of memory).  Within a row the four 16-byte chunks are XOR-swizzled with bits 2-3
+    //      of the row number: rows 4 apart, whose pieces would share banks, read different pieces.  Rows past
+    //      qo_len re-read the last row, chunks past kv_len (last tile of a kv_len that is not a multiple of 64)
+    //      the last chunk: duplicates of valid entries, so neither the products nor the look for a visible key see anything new.
+    const unsigned char* mask_row0 = nullptr;  // uniform: this wave's first mask row
+    unsigned m_goff[2] = {0, 0}, m_goff_last[2] = {0, 0};
+    if constexpr (MASK) {
+        const int row_first = min(m0 + 32 * wave_u, a.M - 1);
+        mask_row0 = static_cast<const unsigned char*>(a.mask) + (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)row_first * a.ms_m;
+        const int last_chunk = ((a.N - 1) % BN) / 16;
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int r = min(16 * e + (lane >> 2), a.M - 1 - row_first);
+            const int chunk = (lane & 3) ^ ((lane >> 4) & 3);  // (bits 2-3 of the row number 16 e + lane / 4)
+            m_goff[e] = (unsigned)(r * (int)a.ms_m + 16 * chunk);
+            m_goff_last[e] = (unsigned)(r * (int)a.ms_m + 16 * min(chunk, last_chunk));
+        }
+    }
+    auto dma_mask = [&](int tile, int slot) {
+        if constexpr (MASK) {
+            const bool cut = ragged && tile == a.nk - 1;
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+                dma16(mask_row0 + (int64_t)tile * BN, cut ? m_goff_last[e] : m_goff[e],
+                      lds0 + F::TOTAL + (slot * kFastWaves + wave_u) * kMaskWaveBytes + 1024 * e);
+        }
+    };
+    // The lane's mask bytes of 16-key slice tp of a staged step: two words, keys 8 g + 4 half .. + 3 for the even and
+    // the odd g of the slice (the keys of score registers 8 (tp & 1) .. + 3 and + 4 .. + 7 of tile tp >> 1).
+    auto mask_words = [&](int slot, int tp, unsigned& even, unsigned& odd) {
+        const unsigned char* row = smem + F::TOTAL + (slot * kFastWaves + wave) * kMaskWaveBytes + l32 * BN + 4 * half;
+        const unsigned* piece = reinterpret_cast<const unsigned*>(row + ((16 * tp) ^ (4 * (l32 & 12))));
+        even = piece[0];
+        odd = piece[2];
+    };
+    // Does the current step's mask tile hold a visible key for this wave's 128-row block?  (The reference skips a
+    // 128 x 64 tile whose mask is False everywhere, attn_qk_int8_per_block.py:33-36.)  Only the path that redoes a
+    // step asks: rows that have seen a key need no answer, their P of a hidden key is 0 either way.  The four
+    // slices of the block lie side by side in the slot; all of them landed before the barrier that opened the
+    // previous phase and are refilled two phases from now at the earliest.
+    auto tile_has_visible_key = [&](int slot) {
+        const uint4* blk = reinterpret_cast<const uint4*>(smem + F::TOTAL + (slot * kFastWaves + 4 * (wave >> 2)) * kMaskWaveBytes);
+        unsigned any = 0;
+#pragma unroll
+        for (int k = 0; k < 4 * kMaskWaveBytes / (64 * 16); k++) {
+            const uint4 w = blk[lane + 64 * k];
+            any |= w.x | w.y | w.z | w.w;
+        }
+        return __builtin_amdgcn_ballot_w64(any != 0) != 0;
+    };
     // ---- fragment read offsets (undoing the swizzle)
     // K: lane (row l32, half) reads chunk half * K_RS/32 + t of its row for k-step t
     int kf_off[F::KSTEPS];
@@ -353,13 +420,15 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const unsigned char* k_fetch = reinterpret_cast<const unsigned char*>(kg);
     const unsigned char* v_fetch = reinterpret_cast<const unsigned char*>(vg);
     int k_tile = 0, v_tile = 0;  // indices of the tiles behind k_fetch / v_fetch
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<1>{}, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
+    sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<1>{}, 0, k_fetch, k_tile, 0, v_fetch, v_tile); });
     if (nsteps > 1) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
-    sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<1>{}, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
+    sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<1>{}, 1, k_fetch, k_tile, 1, v_fetch, v_tile); });
     if (nsteps > 2) { k_fetch += k_tile_bytes; v_fetch += v_tile_bytes; k_tile++; v_tile++; }
     sfor<F::NK>([&](auto ec) { dma_unit(ec, IC<1>{}, 2, k_fetch, k_tile, 2, v_fetch, v_tile); });
     // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
     if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
+    dma_mask(0, 0);
+    dma_mask(min(1, nsteps - 1), 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);
@@ -372,7 +441,9 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // (a row that sees no key at all, qo_len > kv_len under the causal flag, keeps a finite reference
         // point: its exponentials are then exp2(-inf) = 0 and it ends with l = 0)
         m_i = fmaxf((row_pair_max(raw_max) - BIAS) * sc, -1.0e30f);
+        if (MASK) m_i = -INFINITY;  // no visible key seen yet: the first step with one sets the reference point
     }
+    int mslot = 0;  // slot of the current step's mask bytes (step % 3)
 
     // ---- one step.  Each wave alternates a VALU phase (exponentials of its step) and an MFMA phase
     // (Q.K^T of the next step, P.V of this one, with the row sums in the shadow of the matrix
@@ -432,18 +503,31 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             neg_m = -m_i;
         }
         if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
+
         // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
         // instruction.
-        sfor<NDMA>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
+        sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
+        const int mslot_next = mslot == kMaskSlots - 1 ? 0 : mslot + 1;
+        dma_mask(min(step + 2, nsteps - 1), mslot_next == kMaskSlots - 1 ? 0 : mslot_next + 1);  // the mask bytes of step + 2
         vec16 pf[4];
         float lsum = 0.0f;
         const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
+        unsigned mw[2][2] = {{0, 0}, {0, 0}};  // (MASK) the lane's mask bytes of the 16-key slice in work and of the next one
+        if constexpr (MASK) mask_words(mslot, 0, mw[0][0], mw[0][1]);
         auto exp_unit = [&](auto uc) {  // two scores -> two 16-bit P values
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
             const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
+            float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
+            float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
+            if constexpr (MASK) {
+                // P of a hidden key is 0 (mask bytes are 0 / 1).  An overflowed P times 0 is NaN: the row sum then
+                // sends the step into the path that redoes it.
+                if constexpr (w == 0 && tp < 3) mask_words(mslot, tp + 1, mw[(tp + 1) & 1][0], mw[(tp + 1) & 1][1]);
+                const unsigned word = mw[tp & 1][w >> 1];
+                p0 *= (float)((word >> (16 * (w & 1))) & 0xffu);
+                p1 *= (float)((word >> (16 * (w & 1) + 8)) & 0xffu);
+            }
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;
         };
@@ -478,6 +562,64 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         v4f sum4 = {0.0f, 0.0f, 0.0f, 0.0f};
         unsigned long long large = 0;
         auto redo_if_large = [&]() {
+            if constexpr (MASK) {
+                if (large != 0 && !tile_has_visible_key(mslot)) {
+                    // no visible key for this 128-row block in this tile: the reference skips it.  (Rows without a
+                    // reference point get here every step until they see a key: their P came out inf or NaN.)
+#pragma unroll
+                    for (int tp = 0; tp < 4; tp++)
+#pragma unroll
+                        for (int c = 0; c < 8; c++) pf[tp][c] = (VT)0.0f;
+                    lsum = 0.0f;
+                } else if (large != 0) {
+                    // The reference's own arithmetic (attn_qk_int8_per_block.py:44-62): score = dot * scale, plus -1e6
+                    // where the mask hides the key; a key past kv_len scores exactly -1e6 (K and the mask are read
+                    // as zeros / False there).
+                    // (Its V rows are zeros too: such a key adds exp2(-1e6 - m) to the row sum and nothing to O; here
+                    // its P stays 0 and the row sum gets the term directly.)
+                    float raw = -INFINITY;
+                    float past_end = 0.0f;  // number of the lane's keys of this step that lie past kv_len
+                    sfor<4>([&](auto tc) {
+                        constexpr int tp = decltype(tc)::value, kt = tp >> 1;
+                        unsigned ev, od;
+                        mask_words(mslot, tp, ev, od);
+#pragma unroll
+                        for (int c = 0; c < 8; c++) {
+                            const int i = 8 * (tp & 1) + c;
+                            const int bits = sbuf[P][kt][i];
+                            const float x = as_f(bits);
+                            const unsigned keep = (((c >> 2) ? od : ev) >> (8 * (c & 3))) & 0xffu;
+                            float sv = __builtin_fmaf(folded ? x - BIAS : x, sc_e, keep ? 0.0f : kMaskedScore);
+                            if (x == -INFINITY) {  // hidden by position, not by the mask: past kv_len
+                                sv = -INFINITY;
+                                past_end += 1.0f;
+                            }
+                            sbuf[P][kt][i] = __builtin_bit_cast(int, sv);
+                            raw = fmaxf(raw, sv);
+                        }
+                    });
+                    if (past_end > 0.0f) raw = fmaxf(raw, kMaskedScore);
+                    const float m_new = fmaxf(m_i, row_pair_max(raw));
+                    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);  // 0 for a row that had no reference point yet
+                    l_i *= alpha;
+                    m_i = m_new;
+#pragma unroll
+                    for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+                    lsum = 0.0f;
+                    sfor<16>([&](auto uc) {
+                        constexpr int u = decltype(uc)::value;
+                        constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
+                        const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
+                        pf[tp][2 * w] = (VT)__builtin_amdgcn_exp2f(as_f(b0) - m_i);
+                        pf[tp][2 * w + 1] = (VT)__builtin_amdgcn_exp2f(as_f(b1) - m_i);
+                        lsum = PVT::dot2_ones(pf[tp], w, lsum);
+                    });
+                    lsum = __builtin_fmaf(past_end, __builtin_amdgcn_exp2f(kMaskedScore - m_i), lsum);
+                }
+                return;
+            }
             if (large != 0) {
                 float raw = -INFINITY;
 #pragma unroll
@@ -588,6 +730,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             __builtin_amdgcn_sched_barrier(0);
         });
         l_i += lsum;
+        mslot = mslot_next;
         if (step + 4 < nsteps) { k_fetch += k_tile_bytes; k_tile++; }  // next iteration fetches K of step+4, V of step+3
         if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
         __builtin_amdgcn_s_setprio(0);

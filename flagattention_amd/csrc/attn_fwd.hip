@@ -482,6 +482,8 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     else if (p.causal) mode = MODE_CAUSAL;
     const bool fast = p.mask_kind == SAGE_MASK_NONE && (!p.causal || p.qo_len <= p.kv_len);
     if (fast) return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
+    if (p.mask_kind == SAGE_MASK_BOOL && attn::fast_serves_mask(a))
+        return attn::launch_fast_masked(a, (int)p.head_dim, p.v_dtype, stream);
     if (p.head_dim == 128) {
         return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)
                                       : launch_mode<128, _Float16>(a, mode, stream);

@@ -1,5 +1,6 @@
 // SageAttention forward for gfx950, pipelined kernel: the int8 Q, K instances of attn_fast_kernel.h.
-// They serve every call without a mask tensor (causal only with qo_len <= kv_len; any kv_len), under the
+// They serve every call without a mask tensor (causal only with qo_len <= kv_len; any kv_len) and bool mask tensors
+// with 16-byte aligned rows, under the
 // arithmetic contract of FlagAttention src/flag_attn/sage_attention/attn_qk_int8_per_block.py:20-127
 // (per-block scales, base-2 online softmax, lse = log2(l) + m).
 #include "attn_fast_kernel.h"
@@ -20,7 +21,30 @@ int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
     return check_launch("sage_attn_fwd_fast_kernel");
 }
 
+template <int D, typename VT>
+int launch_masked(const AttnArgs& a, hipStream_t stream) {
+    AttnArgs b = a;
+    const int nq2 = (a.M + kFastRows - 1) / kFastRows;
+    b.total_wg = (int)((int64_t)a.total_wg / a.nq * nq2);
+    dim3 grid((unsigned)b.total_wg), block(kFastThreads);
+    hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1, true>), grid, block, 0, stream, b, nq2);
+    return check_launch("sage_attn_fwd_fast_kernel (bool mask)");
+}
+
 }  // namespace
+
+// A bool mask tensor the pipelined kernel can stage with 16-byte loads: contiguous along the keys, every row start
+// 16-byte aligned, kv_len a multiple of 16 (so that no load reaches past the end of a row), no causal flag on top.
+bool fast_serves_mask(const AttnArgs& a) {
+    return a.mask != nullptr && !a.causal && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 && a.ms_b % 16 == 0 &&
+           a.ms_h % 16 == 0 && a.ms_m % 16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 26) && a.N % 16 == 0;
+}
+
+int launch_fast_masked(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream) {
+    if (head_dim == 128)
+        return v_dtype == SAGE_BF16 ? launch_masked<128, __bf16>(a, stream) : launch_masked<128, _Float16>(a, stream);
+    return v_dtype == SAGE_BF16 ? launch_masked<64, __bf16>(a, stream) : launch_masked<64, _Float16>(a, stream);
+}
 
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream) {
     causal = causal || (a.N % BN) != 0;  // the instance that can hide keys also serves a ragged last tile

@@ -74,7 +74,7 @@ int sage_per_block_int8(const sage_quant_params* p, void* stream);
  *   out          out_dtype (SAGE_F16 / SAGE_BF16 / SAGE_F32), own strides
  *   lse          optional [B, Hq, M] fp32 contiguous, base-2 log-sum-exp (:124-127); NULL = none
  *   mask         optional [B, Hq, M, N] through 4 strides (elements, 0 = broadcast);
- *                SAGE_MASK_BOOL: 1 byte per element, non-zero = keep (:33-36,48);
+ *                SAGE_MASK_BOOL: 1 byte per element, 1 = keep, 0 = hide (:33-36,48); other byte values are not allowed;
  *                SAGE_MASK_F32: additive (:38,50)
  *   causal       non-zero adds the bottom-right aligned causal mask n <= m + (N - M), handled
  *                like a bool mask (tiles that are entirely masked are skipped)

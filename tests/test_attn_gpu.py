@@ -234,6 +234,69 @@ def test_row_maximum_that_moves_between_tiles_other_paths(pattern, path, gpu_dev
     torch.testing.assert_close(lse.cpu()[rows], expected_lse[rows], atol=6e-3, rtol=1e-5)
 
 
+def _mask_case(kind, b, h, m, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "random":  # 70 % visible, per (batch, head)
+        return torch.rand(b, h, m, n, generator=g) > 0.3
+    if kind == "broadcast":  # one mask for every batch and head
+        return torch.rand(1, 1, m, n, generator=g) > 0.5
+    rows, cols = torch.arange(m)[:, None], torch.arange(n)[None, :]
+    if kind == "window":  # sliding window: leading tiles without a visible key, rows that start seeing keys at different steps
+        return ((cols <= rows + 40) & (cols >= rows - 90))[None, None].expand(1, 1, m, n)
+    if kind == "holes":  # rows that see nothing at all, rows hidden in some tiles only, a whole 128-row block without keys in a tile
+        mask = torch.rand(b, h, m, n, generator=g) > 0.4
+        mask[:, :, 5] = False
+        mask[:, :, min(77, m - 1), : n // 2] = False
+        mask[:, :, 130:200, 64:128] = False
+        mask[:, :, :128, 128:192] = False
+        mask[:, 0, 256:, : 3 * (n // 4)] = False
+        return mask
+    if kind == "none_visible":
+        return torch.zeros(1, 1, m, n, dtype=torch.bool)
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["random", "broadcast", "window", "holes", "none_visible"])
+@pytest.mark.parametrize("d,vdtype", [(128, torch.bfloat16), (64, torch.float16)])
+@pytest.mark.parametrize("m,n", [(300, 512), (129, 80), (600, 1040), (64, 64)])
+def test_bool_masks_with_aligned_rows(kind, d, vdtype, m, n, gpu_device):
+    """Bool mask tensors whose rows are 16-byte aligned (kv_len a multiple of 16) take the pipelined kernel: checked
+    against the oracle's tile arithmetic, which keeps the reference's -1e6 for hidden keys (a row without a
+    visible key in an unskipped tile is a softmax over its hidden scores, not NaN) and its skipping of 128 x 64
+    tiles without a visible key; grouped heads, ragged query and key lengths, masks broadcast over batch and heads."""
+    b, hq, hkv = 2, 4, 2
+    q8, qs, k8, ks, v = _quantized(41, b, hq, hkv, m, n, d, vdtype)
+    mask = _mask_case(kind, b, hq, m, n, 7)
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask.to(gpu_device), return_lse=True, output_dtype=torch.float32)
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, attn_mask=mask)
+    assert bool(torch.isfinite(o).all())
+    if kind == "none_visible":  # every tile skipped: zero rows, lse = -inf
+        assert float(expected.abs().max()) == 0.0 and float(o.abs().max()) == 0.0
+    else:
+        _gate(o, expected, kind)
+    normal = expected_lse > -1.0e5  # rows that saw a key; the others: -inf (every tile skipped) or about -1e6
+    assert torch.equal(torch.isneginf(lse.cpu()), torch.isneginf(expected_lse))
+    torch.testing.assert_close(lse.cpu()[normal], expected_lse[normal], atol=6e-3, rtol=1e-4)
+    hidden = ~normal & torch.isfinite(expected_lse)
+    torch.testing.assert_close(lse.cpu()[hidden], expected_lse[hidden], atol=1.0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("pattern", sorted(_SCALE_PATTERNS))
+def test_bool_mask_with_row_maximum_that_moves(pattern, gpu_device):
+    m, n = 320, 768
+    q8, qs, k8, ks, v = _quantized(43, 1, 2, 1, m, n, 128, torch.bfloat16)
+    ks2 = ks.clone()
+    for j in range(ks2.shape[-1]):
+        ks2[..., j] *= _SCALE_PATTERNS[pattern](j)
+    mask = _mask_case("holes", 1, 2, m, n, 9)
+    o, lse = _run(gpu_device, q8, qs, k8, ks2, v, attn_mask=mask.to(gpu_device), return_lse=True, output_dtype=torch.float32)
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks2, attn_mask=mask)
+    assert bool(torch.isfinite(o).all())
+    _gate(o, expected, pattern)
+    normal = expected_lse > -1.0e5
+    torch.testing.assert_close(lse.cpu()[normal], expected_lse[normal], atol=6e-3, rtol=1e-5)
+
+
 @pytest.mark.parametrize("n", [64, 192, 320])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_odd_step_counts_and_output_dtypes(n, out_dtype, gpu_device):
