@@ -211,9 +211,15 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
     // The loads are written in assembly: the compiler would otherwise wait for every outstanding one
     // before each LDS read that follows.  Completion is tracked by hand with s_waitcnt vmcnt.
+    // INVARIANT: m0 (the LDS address register of the load) is written here behind the compiler's back: it cannot be
+    // named as a clobber.  That is sound only while the compiler itself never keeps a value in m0 in this kernel;
+    // on gfx950 it would do so for s_movrel / v_movrel (registers indexed by a run-time value), LDS-direct and GWS
+    // instructions and s_sendmsg, none of which this kernel gives it a reason to use (every register array is
+    // indexed by compile-time constants).  tests/test_host_cpu.py compiles this file to assembly and fails if
+    // anything but these moves mentions m0.
     auto dma16 = [](const unsigned char* base, unsigned voff, unsigned lds_addr) {
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");  // (m0 cannot be named as a clobber; nothing else in this kernel uses it)
+                     :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");
     };
     // The last tile of a kv_len that is not a multiple of 64 (CAUSAL instance only): rows past the end
     // re-read the last valid row (finite values under hidden scores), through per-lane offsets of their own.

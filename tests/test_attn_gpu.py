@@ -527,3 +527,31 @@ def test_repeated_calls_are_bit_identical(causal, gpu_device):
         for _ in range(20):
             assert torch.equal(sa.sage_attention(a8, b8, v2, as_, bs, output_dtype=dt, causal=causal)[0], first)
             assert torch.equal(flag_attn.flash_attention(q2, k2, v2, causal), dense_first)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("vdtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("variant", ["plain", "causal", "ragged", "bool_mask"])
+def test_every_pipelined_instance_repeats_and_matches_the_oracle(d, vdtype, variant, gpu_device):
+    """Each instance of the pipelined kernel (head_dim 64 / 128, fp16 / bf16 V, with and without hidden keys,
+    with a staged bool mask): ten calls give the same bits as the first, and the first agrees with the oracle.
+    The kernel's direct-to-LDS loads address LDS through a register the compiler does not know is written: a
+    compiler-made use of it would show here as a wrong or unstable result."""
+    n = 1000 if variant == "ragged" else 1024
+    q8, qs, k8, ks, v = _quantized(51, 2, 4, 2, 700, n, d, vdtype)
+    kw, okw = {}, {}
+    if variant == "causal":
+        kw = okw = {"causal": True}
+    elif variant == "bool_mask":
+        mask = _mask_case("random", 2, 4, 700, n, 3)
+        kw, okw = {"attn_mask": mask.to(gpu_device)}, {"attn_mask": mask}
+    first = _run(gpu_device, q8, qs, k8, ks, v, return_lse=True, output_dtype=vdtype, **kw)
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, **okw)
+    _gate(first[0], expected, variant)
+    torch.testing.assert_close(first[1].cpu(), expected_lse, atol=6e-3, rtol=1e-4)
+    dev = [t.to(gpu_device) for t in (q8, k8, v, qs, ks)]
+    from flag_attn import sage_attention as sa
+
+    for _ in range(10):
+        again = sa.sage_attention(dev[0], dev[1], dev[2], dev[3], dev[4], return_lse=True, output_dtype=vdtype, **kw)
+        assert torch.equal(again[0], first[0]) and torch.equal(again[1], first[1])

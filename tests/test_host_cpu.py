@@ -192,3 +192,25 @@ def test_benchmark_rows_record_format(tmp_path, monkeypatch):
     assert R.baseline_name(torch.bfloat16) == "torch_sdpa_plus_bfloat16_cast"
     if not torch.cuda.is_available():
         assert R.main(["--seq-lens", "128"]) == 1
+
+
+@pytest.mark.skipif(not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
+def test_only_the_lds_load_sequence_touches_m0(tmp_path):
+    """The pipelined attention kernel sets m0 in inline assembly, which the compiler cannot be told about.  Compile
+    its translation units to assembly and check that m0 appears nowhere else: only as the destination of the
+    s_mov_b32 that precedes each direct-to-LDS load."""
+    import re
+    import subprocess
+
+    csrc = os.path.join(ROOT, "flagattention_amd", "csrc")
+    for unit in ("attn_fwd_fast.hip", "flash_fwd.hip"):
+        out = tmp_path / (unit + ".s")
+        subprocess.run(["/opt/rocm/bin/hipcc", "-O3", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=off", "-Xclang",
+                        "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", "-o", str(out),
+                        os.path.join(csrc, unit)], check=True, capture_output=True, timeout=600)
+        mentions = [ln.strip() for ln in out.read_text().splitlines() if re.search(r"\bm0\b", ln.split(";")[0])]
+        assert mentions, "expected the direct-to-LDS load sequence in " + unit
+        other = [ln for ln in mentions if not re.fullmatch(r"s_mov_b32 m0, s\d+", ln)]
+        assert not other, other[:5]
+        loads = sum(1 for ln in out.read_text().splitlines() if ln.strip().startswith("global_load_lds_dwordx4"))
+        assert loads == len(mentions)
