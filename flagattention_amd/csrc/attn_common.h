@@ -38,6 +38,7 @@ struct AttnArgs {
     int32_t out_dt, causal;
     int32_t total_wg;
     int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
+    int32_t mask_dt;   // storage type of an additive mask (SAGE_F32 / SAGE_F16 / SAGE_BF16)
     float lse_mul;     // factor on the base-2 log-sum-exp on its way out (1: as is; ln 2: natural log)
     float qk_scale;    // 16-bit Q and K only: sm_scale * log2(e), the one scale of every score (q/k point at 16-bit data)
 };

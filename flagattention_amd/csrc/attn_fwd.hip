@@ -56,6 +56,22 @@ __device__ __forceinline__ float xhalf_sum(float x) {
     return (threadIdx.x & 32) ? (o + x) : (x + o);  // same operand order in both halves
 }
 
+// Additive mask entries as fp32, whatever the mask's storage type (fp32, fp16 or bf16: a.mask_dt).
+__device__ __forceinline__ float mask_entry(const AttnArgs& a, int64_t idx) {
+    if (a.mask_dt == SAGE_F32) return static_cast<const float*>(a.mask)[idx];
+    if (a.mask_dt == SAGE_BF16) return (float)static_cast<const __bf16*>(a.mask)[idx];
+    return (float)static_cast<const _Float16*>(a.mask)[idx];
+}
+__device__ __forceinline__ float4 mask_run4(const AttnArgs& a, int64_t idx) {  // four consecutive, naturally aligned entries
+    if (a.mask_dt == SAGE_F32) return *reinterpret_cast<const float4*>(static_cast<const float*>(a.mask) + idx);
+    const uint2 w = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.mask) + idx);
+    if (a.mask_dt == SAGE_BF16)
+        return make_float4(__builtin_bit_cast(float, w.x << 16), __builtin_bit_cast(float, w.x & 0xffff0000u),
+                           __builtin_bit_cast(float, w.y << 16), __builtin_bit_cast(float, w.y & 0xffff0000u));
+    return make_float4((float)__builtin_bit_cast(_Float16, (uint16_t)(w.x & 0xffffu)), (float)__builtin_bit_cast(_Float16, (uint16_t)(w.x >> 16)),
+                       (float)__builtin_bit_cast(_Float16, (uint16_t)(w.y & 0xffffu)), (float)__builtin_bit_cast(_Float16, (uint16_t)(w.y >> 16)));
+}
+
 template <int D, typename VT, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) {
     using T = Tile<D>;
@@ -220,7 +236,7 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
             const int nb = run_start(step, r);
             if (nb + 3 < a.N) {
                 if (MODE == MODE_MASK_BOOL) mw[r] = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(a.mask) + mrow + nb);
-                else mf[r] = *reinterpret_cast<const float4*>(static_cast<const float*>(a.mask) + mrow + nb);
+                else mf[r] = mask_run4(a, mrow + nb);
             }
         }
     };
@@ -288,7 +304,7 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
                             float mf = 0.0f;
                             if (inb) {
                                 if (MODE == MODE_MASK_BOOL) mb = static_cast<const uint8_t*>(a.mask)[mrow + (int64_t)n * a.ms_n] != 0;
-                                else mf = static_cast<const float*>(a.mask)[mrow + (int64_t)n * a.ms_n];
+                                else mf = mask_entry(a, mrow + (int64_t)n * a.ms_n);
                             }
                             entry(kt, 4 * g + e, n, inb, mb, mf, true);
                         }
@@ -464,8 +480,11 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     a.groups = (int)(p.heads_q / p.heads_kv);
     a.out_dt = p.out_dtype; a.causal = p.causal ? 1 : 0;
     a.lse_mul = 1.0f;
+    const bool additive = p.mask_kind == SAGE_MASK_F32 || p.mask_kind == SAGE_MASK_F16 || p.mask_kind == SAGE_MASK_BF16;
+    a.mask_dt = p.mask_kind == SAGE_MASK_F16 ? SAGE_F16 : p.mask_kind == SAGE_MASK_BF16 ? SAGE_BF16 : SAGE_F32;
     if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_n == 1) {
-        const int64_t align = p.mask_kind == SAGE_MASK_BOOL ? 4 : 16, esz = p.mask_kind == SAGE_MASK_BOOL ? 1 : 4;
+        // runs of four entries are read with one load where they are naturally aligned
+        const int64_t esz = p.mask_kind == SAGE_MASK_BOOL ? 1 : dtype_bytes(a.mask_dt), align = 4 * esz;
         a.mask_vec = ((uintptr_t)p.mask % align) == 0 && (p.mask_stride_b * esz) % align == 0 &&
                      (p.mask_stride_h * esz) % align == 0 && (p.mask_stride_m * esz) % align == 0;
     }
@@ -478,7 +497,7 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
     a.total_wg = (int)total;
     int mode = MODE_PLAIN;
     if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
-    else if (p.mask_kind == SAGE_MASK_F32) mode = MODE_MASK_F32;
+    else if (additive) mode = MODE_MASK_F32;
     else if (p.causal) mode = MODE_CAUSAL;
     const bool fast = p.mask_kind == SAGE_MASK_NONE && (!p.causal || p.qo_len <= p.kv_len);
     if (fast) return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);

@@ -109,9 +109,13 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
             m = attn_mask
             if m.dtype == torch.bool:
                 p.mask_kind = _lib.MASK_BOOL
+            elif m.dtype == torch.float16:
+                p.mask_kind = _lib.MASK_F16
+            elif m.dtype == torch.bfloat16:
+                p.mask_kind = _lib.MASK_BF16
             else:
                 p.mask_kind = _lib.MASK_F32
-                if m.dtype != torch.float32:
+                if m.dtype != torch.float32:  # (float64 or integer masks: the kernel adds fp32 values)
                     m = m.float()
             m = m.expand(b, h_qo, qo_len, kv_len)
             mask_keepalive = m

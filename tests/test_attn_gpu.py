@@ -555,3 +555,18 @@ def test_every_pipelined_instance_repeats_and_matches_the_oracle(d, vdtype, vari
     for _ in range(10):
         again = sa.sage_attention(dev[0], dev[1], dev[2], dev[3], dev[4], return_lse=True, output_dtype=vdtype, **kw)
         assert torch.equal(again[0], first[0]) and torch.equal(again[1], first[1])
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("m,n", [(129, 257), (300, 512)])
+def test_additive_masks_of_other_float_types(mask_dtype, m, n, gpu_device):
+    """Additive masks stored as fp16 / bf16 are read as they are (no fp32 copy of the mask is made); other types
+    are converted by the wrapper.  The values added are the fp32 images of the stored entries."""
+    q8, qs, k8, ks, v = _quantized(61, 1, 2, 2, m, n, 64, torch.float16)
+    g = torch.Generator().manual_seed(8)
+    mask = (torch.randn(1, 2, m, n, generator=g) * 3.0).to(mask_dtype)
+    mask[..., ::5] = -30.0
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask.to(gpu_device), return_lse=True, output_dtype=torch.float32)
+    expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, attn_mask=mask.float())
+    _gate(o, expected)
+    torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
