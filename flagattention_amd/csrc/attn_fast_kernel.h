@@ -57,7 +57,11 @@ constexpr float kBias = 12582912.0f;
 // exp2(fma(kBias + dot, sc, -(kBias * sc + m))) loses ulp(kBias * sc) / 2 in the exponent; above this
 // product the bias is subtracted explicitly instead.
 constexpr float kBiasFoldLimit = 8192.0f;
-constexpr float kSumLimit = 8192.0f;  // a lane's 32 P of one step sum to less than this, or the step is redone
+// A lane's 32 P of one step sum to less than this, or the step is redone.  fp16 P: no P may pass 65504.  bf16 P has
+// the exponent range of fp32: the limit only keeps 2^60 * |V| * kv_len and the row sums far inside that range, so a
+// row maximum may run up to 60 log2 units ahead of the row's reference point before a step has to be redone.
+template <typename VT> constexpr float sum_limit() { return 32768.0f; }
+template <> constexpr float sum_limit<__bf16>() { return 0x1p60f; }
 constexpr int kFastWaves = 8;                     // waves per workgroup, 32 query rows each
 constexpr int kFastThreads = 64 * kFastWaves;
 constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
@@ -122,6 +126,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr float BIAS = INT8 ? kBias : 0.0f;  // what the bits of a fresh score accumulator read as a float
     using PVT = PV<VT>;
     using vec16 = typename PVT::vec;
+    constexpr float kSumLimit = sum_limit<VT>();
     __shared__ __attribute__((aligned(16))) unsigned char smem[F::TOTAL + (MASK ? kMaskBytes : 0)];
 
 
@@ -496,9 +501,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // is redone against its true maximum: see redo_if_large below.
         float neg_m;
         const bool folded = !INT8 || kBias * sc < kBiasFoldLimit;
-        if (folded) {
-            neg_m = __builtin_fmaf(-BIAS, sc, -m_i);
-        } else {
+        if (!folded) {
 #pragma unroll
             for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -506,8 +509,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                     const int bits = sbuf[P][kt][i];
                     sbuf[P][kt][i] = __builtin_bit_cast(int, as_f(bits) - kBias);
                 }
-            neg_m = -m_i;
         }
+        neg_m = folded ? __builtin_fmaf(-BIAS, sc, -m_i) : -m_i;
         if (!live) neg_m = -INFINITY;  // padding step: every P is exp2(-inf) = 0
 
         // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
