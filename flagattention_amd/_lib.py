@@ -65,6 +65,7 @@ EXPORTS = (
     "sage_per_block_int8_smooth_k",
     "sage_attn_fwd",
     "sage_flash_attn_fwd",
+    "sage_flash_total_attention",
     "sage_k_mean",
     "sage_k_mean_workspace_bytes",
     "sage_k_mean_noalloc",
@@ -99,6 +100,8 @@ def load():
     lib.sage_attn_fwd.restype = ctypes.c_int
     lib.sage_flash_attn_fwd.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p]
     lib.sage_flash_attn_fwd.restype = ctypes.c_int
+    lib.sage_flash_total_attention.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.sage_flash_total_attention.restype = ctypes.c_int
     lib.sage_k_mean_workspace_bytes.argtypes = [c_i64] * 4
     lib.sage_k_mean_workspace_bytes.restype = c_i64
     lib.sage_k_mean.argtypes = [ctypes.POINTER(SageTensor), c_i32, ctypes.c_void_p, c_i32, c_i64, c_i64, c_i64,

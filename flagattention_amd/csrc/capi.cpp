@@ -144,9 +144,24 @@ extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
     return launch_attn(*p, (hipStream_t)stream);
 }
 
+static int check_flash_params(const sage_flash_params* p, bool forward);
+
 extern "C" int sage_flash_attn_fwd(const sage_flash_params* p, void* stream) {
+    if (int rc = check_flash_params(p, true)) return rc;
+    return launch_flash_attn(*p, (hipStream_t)stream);
+}
+
+extern "C" int sage_flash_total_attention(const sage_flash_params* p, const float* log_normalizer, float* total_attention,
+                                          void* stream) {
+    if (int rc = check_flash_params(p, false)) return rc;
+    if (!log_normalizer || !total_attention)
+        return fail(SAGE_E_INVALID, "sage_flash_total_attention: null log_normalizer or total_attention");
+    return launch_flash_total_attention(*p, log_normalizer, total_attention, (hipStream_t)stream);
+}
+
+static int check_flash_params(const sage_flash_params* p, bool forward) {
     if (!p) return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: null params");
-    if (!p->q.ptr || !p->k.ptr || !p->v.ptr || !p->out.ptr)
+    if (!p->q.ptr || !p->k.ptr || (forward && (!p->v.ptr || !p->out.ptr)))
         return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: null tensor pointer");
     if (p->head_dim != 64 && p->head_dim != 128)
         return fail(SAGE_E_UNSUPPORTED, "sage_flash_attn_fwd: head_dim %lld not supported (64 or 128)",
@@ -158,16 +173,16 @@ extern "C" int sage_flash_attn_fwd(const sage_flash_params* p, void* stream) {
                     (long long)p->heads_q, (long long)p->heads_kv);
     if (p->dtype != SAGE_F16 && p->dtype != SAGE_BF16)
         return fail(SAGE_E_UNSUPPORTED, "sage_flash_attn_fwd: q, k, v must be fp16 or bf16");
-    if (!float_dtype_ok(p->out_dtype)) return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: bad out_dtype %d", p->out_dtype);
+    if (forward && !float_dtype_ok(p->out_dtype)) return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: bad out_dtype %d", p->out_dtype);
     if (!(p->sm_scale > 0.0f) || !(p->sm_scale < 3.0e38f))
         return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: sm_scale must be positive and finite");
     auto misaligned = [](const sage_tensor& t, int esz) {
         return ((uintptr_t)t.ptr % 16) != 0 || (t.stride_b * esz) % 16 != 0 || (t.stride_h * esz) % 16 != 0 ||
                (t.stride_n * esz) % 16 != 0;
     };
-    if (misaligned(p->q, 2) || misaligned(p->k, 2) || misaligned(p->v, 2))
+    if (misaligned(p->q, 2) || misaligned(p->k, 2) || (forward && misaligned(p->v, 2)))
         return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: q/k/v rows must be 16-byte aligned");
-    if (misaligned(p->out, dtype_bytes(p->out_dtype)))
+    if (forward && misaligned(p->out, dtype_bytes(p->out_dtype)))
         return fail(SAGE_E_INVALID, "sage_flash_attn_fwd: out rows must be 16-byte aligned");
-    return launch_flash_attn(*p, (hipStream_t)stream);
+    return SAGE_OK;
 }

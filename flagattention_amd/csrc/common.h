@@ -27,5 +27,6 @@ int launch_smooth_quant(const sage_quant_params& p, void* km_out, float* q_dot_k
 int static_scratch(void** out);
 int launch_attn(const sage_attn_params& p, hipStream_t stream);
 int launch_flash_attn(const sage_flash_params& p, hipStream_t stream);
+int launch_flash_total_attention(const sage_flash_params& p, const float* log_normalizer, float* total, hipStream_t stream);
 
 }  // namespace sage

@@ -5,8 +5,8 @@
 Built here: the forward pass for fp16 / bf16, head_dim 64 or 128 (16 and 32, which the reference also
 takes, flash.py:43, run through zero-padded copies of q, k, v at head_dim 64), grouped K/V heads, the
 causal flag for any qo_len / kv_len (bottom-right aligned, flash.py:53-54), ``sm_scale`` and the
-natural-log log normalizer (flash.py:503-506).  Not built: dropout, the total attention and the
-backward pass; a call that asks for one of them raises instead of computing something else.
+natural-log log normalizer (flash.py:503-506), and the total attention (flash.py:142-157, total.py).  Not built:
+dropout and the backward pass; a call that asks for one of them raises instead of computing something else.
 """
 from __future__ import annotations
 
@@ -29,8 +29,9 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
               return_log_normalizer=False, return_total_attention=False, return_seed_offset=False):
     """O = softmax(sm_scale * Q K^T [causal]) V, and optionally logsumexp(sm_scale * Q K^T) per query.
 
-    Returns ``o`` alone, or the reference's 5-tuple ``(o, log_normalizer, None, None, None)`` when an
-    extra output is asked for (flash.py:170-180).
+    Returns ``o`` alone, or the reference's 5-tuple ``(o, log_normalizer, total_attention, None, None)`` when an
+    extra output is asked for (flash.py:170-180): ``log_normalizer`` ``[B, H, M]`` and ``total_attention``
+    ``[B, H, N]`` (the attention every key receives, summed over the queries) in fp32, None where not asked for.
     """
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be (batch, heads, sequence, head_dim) tensors")
@@ -45,8 +46,6 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
         raise ValueError("batch and sequence sizes of q, k, v do not match")
     if dropout_p != 0.0 or return_seed_offset:
         raise NotImplementedError("flagattention_amd.flash.attention: dropout is not built")
-    if return_total_attention:
-        raise NotImplementedError("flagattention_amd.flash.attention: the total attention is not built")
     if D not in (16, 32, 64, 128):
         raise NotImplementedError(f"flagattention_amd.flash.attention: head_dim {D} is not built (16, 32, 64 or 128)")
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -68,7 +67,8 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     o = torch.empty_like(q)  # (the reference allocates the same way, flash.py:84-90)
     if not rows_aligned(o):
         o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    L = torch.empty((B, H, M), dtype=torch.float32, device=q.device) if return_log_normalizer else None
+    need_L = return_log_normalizer or return_total_attention
+    L = torch.empty((B, H, M), dtype=torch.float32, device=q.device) if need_L else None
 
     p = _lib.FlashParams()
     p.q, p.k, p.v, p.out = (tensor_desc(t, True) for t in (q, k, v, o))
@@ -80,8 +80,13 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     lib = _lib.load()
     with torch.cuda.device(q.device):
         _lib.check(lib.sage_flash_attn_fwd(p, current_stream_ptr(q.device)), "sage_flash_attn_fwd")
+        tot = None
+        if return_total_attention:
+            tot = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+            _lib.check(lib.sage_flash_total_attention(p, L.data_ptr(), tot.data_ptr(), current_stream_ptr(q.device)),
+                       "sage_flash_total_attention")
     if D < 64:
         o = o[..., :D].contiguous()
-    if return_log_normalizer:
-        return o, L, None, None, None
+    if return_log_normalizer or return_total_attention:
+        return o, (L if return_log_normalizer else None), tot, None, None
     return o

@@ -169,6 +169,17 @@ typedef struct sage_flash_params {
 
 int sage_flash_attn_fwd(const sage_flash_params* p, void* stream);
 
+/*
+ * Total attention of the same operator: total_attention[b, h, n] = sum over the queries m of
+ * softmax(sm_scale * Q K^T [+ causal])[m, n], recomputed from Q, K and the log normalizer that
+ * sage_flash_attn_fwd returned for the same arguments (src/flag_attn/total.py:22-160, called from
+ * flash.py:142-157).  v, out and out_dtype of the params are not used.
+ *   log_normalizer   [B, Hq, M] fp32 contiguous (natural log), as written by sage_flash_attn_fwd
+ *   total_attention  [B, Hq, N] fp32 contiguous, written in full
+ */
+int sage_flash_total_attention(const sage_flash_params* p, const float* log_normalizer, float* total_attention,
+                               void* stream);
+
 /* Message describing the last non-zero status returned on this thread ("" if none). */
 const char* sage_hip_last_error(void);
 

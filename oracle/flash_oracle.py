@@ -13,7 +13,9 @@ INFRASTRUCTURE ONLY: nothing in the shipped package may import this module (it i
 What pins it (tests/test_oracle_pins.py): it reduces to ``F.scaled_dot_product_attention`` for the
 non-causal case and for causal with M == N; for M != N and for rows that see no key it is checked
 against a brute-force loop over (query, key) pairs on tiny inputs; the log normalizer against
-``log(sum(exp(.)))`` computed in float64.
+``log(sum(exp(.)))`` computed in float64; the total attention against the same brute-force loop
+(sum over the queries of exp(score - log normalizer)) and against two invariants: it sums to the number of
+queries that see a key, and with V = identity the output's column sums are the total attention.
 """
 from __future__ import annotations
 
@@ -22,8 +24,10 @@ import math
 import torch
 
 
-def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False, upcast=True):
-    """q [B,H,M,D], k/v [B,Hk,N,D] (CPU).  Returns o (input dtype) or (o, log_normalizer fp32 [B,H,M])."""
+def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False, upcast=True, return_total_attention=False):
+    """q [B,H,M,D], k/v [B,Hk,N,D] (CPU).  Returns o (input dtype), or (o, log_normalizer fp32 [B,H,M]), or with
+    return_total_attention (o, log_normalizer or None, total_attention fp32 [B,H,N]): the column sums of P over
+    the queries (testing/flash.py:66-67)."""
     input_dtype = q.dtype
     if upcast:
         q, k, v = q.float(), k.float(), v.float()
@@ -46,6 +50,8 @@ def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False,
     if causal:
         p = torch.where(visible, p, 0.0)  # also turns the NaN rows of queries that see no key into zeros
     o = (p.to(v.dtype) @ v).to(input_dtype)
+    if return_total_attention:
+        return o, log_normalizer, p.sum(dim=-2)
     return (o, log_normalizer) if return_log_normalizer else o
 
 

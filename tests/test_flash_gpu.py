@@ -112,8 +112,6 @@ def test_unbuilt_features_raise(gpu_device):
     with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q, k, v, dropout_p=0.1)
     with pytest.raises(NotImplementedError):
-        flag_attn.flash_attention(q, k, v, return_total_attention=True)
-    with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q[..., :48], k[..., :48], v[..., :48])
     with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q.requires_grad_(), k, v)
@@ -256,3 +254,33 @@ def test_long_sequence_against_chunked_fp32(causal, gpu_device):
         worst_l = max(worst_l, (L[:, :, rows] - torch.logsumexp(s, dim=-1)).abs().max().item())
     assert worst <= 2 * yard + 1e-5, (worst, yard)
     assert worst_l <= 2e-3, worst_l
+
+
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", [
+    (2, 4, 4, 512, 612, 128), (2, 4, 2, 1024, 1034, 64), (2, 4, 4, 1000, 1000, 32), (2, 4, 1, 1001, 1096, 64),
+    (1, 2, 2, 1096, 1001, 128), (1, 2, 2, 2048, 2058, 16), (1, 3, 3, 33, 200, 64), (1, 2, 1, 300, 31, 128),
+])
+def test_total_attention_against_reference_rule(B, Hq, Hk, M, N, D, causal, dtype, order, gpu_device):
+    """The auxiliary outputs under the reference's own acceptance rule (tests/flag_attn/test_flash_attention.py:
+    255-296: the test matrix there, both storage orders, fp16 / bf16, and the causal flag on top): the total
+    attention may deviate from the fp32 closed form at most twice as far as the 16-bit closed form does."""
+    import flag_attn
+
+    q, k, v = _inputs(11, B, Hq, Hk, M, N, D, dtype, order=order)
+    o, L, tot, seed, offset = flag_attn.flash_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), causal,
+                                                        return_log_normalizer=True, return_total_attention=True)
+    torch.cuda.synchronize()
+    assert seed is None and offset is None and tot.shape == (B, Hq, N) and tot.dtype == torch.float32
+    o_ref, L_ref, tot_ref = FO.attention(q, k, v, causal, return_log_normalizer=True, return_total_attention=True, upcast=True)
+    _, _, tot_16 = FO.attention(q, k, v, causal, return_total_attention=True, upcast=False)
+    yard = FO.max_diff(tot_16, tot_ref)
+    got = FO.max_diff(tot.cpu(), tot_ref)
+    assert got <= 2 * yard + 1e-5, f"total attention: max diff {got} against a 16-bit yardstick of {yard}"
+    # every query that sees a key hands out attention 1 in total
+    seeing = M if not causal else sum(1 for m in range(M) if m + (N - M) >= 0)
+    torch.testing.assert_close(tot.sum(-1).cpu(), torch.full((B, Hq), float(seeing)), atol=seeing * 2e-3, rtol=0)
+    only_tot = flag_attn.flash_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), causal, return_total_attention=True)
+    assert only_tot[1] is None and torch.equal(only_tot[2], tot) and torch.equal(only_tot[0], o)

@@ -292,3 +292,34 @@ def test_accuracy_metrics_known_answers():
     # shapes are flattened, 16-bit inputs are compared in fp32 / fp64
     cos, rel, max_abs = O.accuracy_metrics(torch.ones(2, 3, dtype=torch.bfloat16), torch.full((2, 3), 1.5))
     assert abs(cos - 1.0) < 1e-12 and abs(rel - 1.0 / 3.0) < 1e-12 and max_abs == 0.5
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n", [(5, 9), (9, 5), (7, 7)])
+def test_flash_oracle_total_attention(causal, m, n):
+    """Total attention = attention every key receives, summed over the queries: a brute-force loop over
+    (query, key) pairs, and two invariants (it sums to the number of queries that see a key; with V = identity
+    the column sums of the output are the total attention).  A sum over keys instead of queries, a missing causal
+    zero or a head-group mix-up fails one of them."""
+    from oracle import flash_oracle as FO
+
+    g = torch.Generator().manual_seed(100 * m + n)
+    q = torch.randn(2, 4, m, 8, generator=g)
+    k = torch.randn(2, 2, n, 8, generator=g)
+    v = torch.randn(2, 2, n, 8, generator=g)
+    o, lse, tot = FO.attention(q, k, v, causal=causal, sm_scale=0.6, return_log_normalizer=True, return_total_attention=True)
+    assert tot.shape == (2, 4, n) and tot.dtype == torch.float32
+    _, blse = _brute_force_attention(q, k, v, causal, 0.6)
+    want = torch.zeros(2, 4, n, dtype=torch.float64)
+    for b in range(2):
+        for h in range(4):
+            for mm in range(m):
+                for nn in range(n):
+                    if (not causal or nn <= mm + (n - m)) and math.isfinite(float(blse[b, h, mm])):
+                        want[b, h, nn] += math.exp(0.6 * float(q[b, h, mm].double() @ k[b, h // 2, nn].double()) - float(blse[b, h, mm]))
+    torch.testing.assert_close(tot.double(), want, atol=1e-5, rtol=1e-5)
+    seeing = sum(1 for mm in range(m) if (not causal) or mm + (n - m) >= 0)
+    torch.testing.assert_close(tot.sum(-1), torch.full((2, 4), float(seeing)), atol=1e-4, rtol=1e-5)
+    eye = torch.eye(n).expand(2, 2, n, n).contiguous()  # V = identity: o[m, :] = P[m, :]
+    o_eye, _, tot_eye = FO.attention(q, k, eye, causal=causal, sm_scale=0.6, return_total_attention=True)
+    torch.testing.assert_close(o_eye.sum(dim=-2), tot_eye, atol=1e-5, rtol=1e-5)
