@@ -487,14 +487,21 @@ __global__ __launch_bounds__(kStage1Threads) void smooth_stage1_kernel(QuantArgs
 }
 
 __global__ __launch_bounds__(kThreads) void k_mean_final_kernel(KMeanArgs a, int64_t channels) {
-    const int64_t ch = (int64_t)blockIdx.x * kThreads + threadIdx.x;  // (b*H + h) * D + d
+    const int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // (b*H + h) * D + d
     if (ch >= channels) return;
     const int64_t bh = ch / a.D;
     const int d = (int)(ch % a.D);
     const float* p = a.part + bh * a.nchunk * a.D + d;
     float tot = 0.0f;
     int c = 0;
-    for (; c + 8 <= a.nchunk; c += 8) {  // loads issued together, additions kept in chunk order
+    for (; c + 32 <= a.nchunk; c += 32) {  // loads issued together, additions kept in chunk order
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) v[i] = p[(int64_t)(c + i) * a.D];
+#pragma unroll
+        for (int i = 0; i < 32; i++) tot = tot + v[i];
+    }
+    for (; c + 8 <= a.nchunk; c += 8) {
         float v[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) v[i] = p[(int64_t)(c + i) * a.D];
@@ -595,8 +602,9 @@ int k_mean_args(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype, 
 }
 
 int launch_k_mean_final(const KMeanArgs& a, int64_t channels, hipStream_t stream) {
-    const int64_t g2 = (channels + kThreads - 1) / kThreads;
-    hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)g2), dim3(kThreads), 0, stream, a, channels);
+    constexpr int kFinalThreads = 64;  // few channels (B * H * D): one wave per workgroup spreads them over the CUs
+    const int64_t g2 = (channels + kFinalThreads - 1) / kFinalThreads;
+    hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)g2), dim3(kFinalThreads), 0, stream, a, channels);
     return check_launch("k_mean_final_kernel");
 }
 
