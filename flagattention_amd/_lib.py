@@ -64,7 +64,11 @@ EXPORTS = (
     "sage_per_block_int8",
     "sage_per_block_int8_smooth_k",
     "sage_attn_fwd",
+    "sage_attn_fwd_workspace_bytes",
+    "sage_attn_fwd_ws",
     "sage_flash_attn_fwd",
+    "sage_flash_attn_fwd_workspace_bytes",
+    "sage_flash_attn_fwd_ws",
     "sage_flash_total_attention",
     "sage_k_mean",
     "sage_k_mean_workspace_bytes",
@@ -100,6 +104,14 @@ def load():
     lib.sage_attn_fwd.restype = ctypes.c_int
     lib.sage_flash_attn_fwd.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p]
     lib.sage_flash_attn_fwd.restype = ctypes.c_int
+    lib.sage_attn_fwd_workspace_bytes.argtypes = [ctypes.POINTER(AttnParams)]
+    lib.sage_attn_fwd_workspace_bytes.restype = c_i64
+    lib.sage_attn_fwd_ws.argtypes = [ctypes.POINTER(AttnParams), ctypes.c_void_p, c_i64, ctypes.c_void_p]
+    lib.sage_attn_fwd_ws.restype = ctypes.c_int
+    lib.sage_flash_attn_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FlashParams)]
+    lib.sage_flash_attn_fwd_workspace_bytes.restype = c_i64
+    lib.sage_flash_attn_fwd_ws.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p, c_i64, ctypes.c_void_p]
+    lib.sage_flash_attn_fwd_ws.restype = ctypes.c_int
     lib.sage_flash_total_attention.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.sage_flash_total_attention.restype = ctypes.c_int
     lib.sage_k_mean_workspace_bytes.argtypes = [c_i64] * 4

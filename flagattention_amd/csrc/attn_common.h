@@ -15,6 +15,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 constexpr int kThreads = 256;
 constexpr int BM = 128;  // query rows per workgroup (= Q quantization block)
 constexpr int BN = 64;   // keys per step (= K quantization block)
+constexpr int kFastRows = 256;  // query rows per workgroup of the pipelined kernel (attn_fast_kernel.h)
 constexpr float kMasked = -1.0e6f;
 constexpr float kTau = 8.0f;  // log2 of the largest P tolerated before the running maximum is advanced
 
@@ -39,6 +40,11 @@ struct AttnArgs {
     int32_t total_wg;
     int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
     int32_t mask_dt;   // storage type of an additive mask (SAGE_F32 / SAGE_F16 / SAGE_BF16)
+    // Split of the keys over several workgroups per (batch, head, q-block) (never under a mask tensor): workgroup s
+    // of `nsplit` takes steps s * split_steps .. and writes an fp32 partial output and its base-2 log-sum-exp to
+    // out + s * out_split_stride / lse + s * lse_split_stride, which a second kernel combines.  Unsplit: 1, nk, 0, 0.
+    int32_t nsplit, split_steps;
+    int64_t out_split_stride, lse_split_stride;
     float lse_mul;     // factor on the base-2 log-sum-exp on its way out (1: as is; ln 2: natural log)
     float qk_scale;    // 16-bit Q and K only: sm_scale * log2(e), the one scale of every score (q/k point at 16-bit data)
 };
@@ -80,6 +86,15 @@ template <> struct PV<_Float16> {
 // Launches the software-pipelined kernel: no mask tensor, and qo_len <= kv_len when causal.
 // head_dim 64 / 128, V dtype fp16 / bf16.
 int launch_fast(const AttnArgs& a, int head_dim, int v_dtype, bool causal, hipStream_t stream);
+
+// Key split for launches that would leave most compute units idle (split_combine.hip).  plan_key_split: how many
+// workgroups share the keys of one (batch, head, q-block), 1 when the launch fills the chip anyway.
+// apply_key_split turns the arguments of the unsplit launch into those of the split one (partial results in
+// `workspace`, key_split_workspace_bytes large); launch_split_combine writes what the unsplit launch would have.
+int plan_key_split(int64_t batch, int64_t heads_q, int64_t qo_len, int64_t kv_len, bool causal);
+int64_t key_split_workspace_bytes(int nsplit, int64_t batch, int64_t heads_q, int64_t qo_len, int64_t head_dim);
+void apply_key_split(AttnArgs& a, int nsplit, int64_t batch, int head_dim, void* workspace);
+int launch_split_combine(const AttnArgs& split, const AttnArgs& whole, int head_dim, int64_t batch, hipStream_t stream);
 
 // The same kernel under a bool mask tensor, where fast_serves_mask() says so (a.mask set, MODE_MASK_BOOL).
 bool fast_serves_mask(const AttnArgs& a);

@@ -64,7 +64,7 @@ template <typename VT> constexpr float sum_limit() { return 32768.0f; }
 template <> constexpr float sum_limit<__bf16>() { return 0x1p60f; }
 constexpr int kFastWaves = 8;                     // waves per workgroup, 32 query rows each
 constexpr int kFastThreads = 64 * kFastWaves;
-constexpr int kFastRows = 32 * kFastWaves;        // query rows per workgroup
+static_assert(kFastRows == 32 * kFastWaves, "query rows per workgroup");
 constexpr int kFastWgPerCu = 8 / kFastWaves;      // two waves per SIMD either way
 
 // LDS tiles are unpadded ([64 keys][row bytes]) because they are filled by direct-to-LDS loads, which
@@ -138,6 +138,14 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
     const bool paired = CAUSAL && a.causal;
     const int per_head = paired ? (nq2 + 1) / 2 : nq2;  // workgroups per (batch, head)
+    // The keys of one (batch, head, q-block) may be split over `nsplit` workgroups (never under a mask tensor).  A
+    // workgroup then sees the problem that starts at its first key: kv_len, the number of tiles and the causal
+    // limits below all count from there, and its steps end where the next workgroup's begin.
+    const int nsplit = MASK ? 1 : a.nsplit;
+    const int split = wg % nsplit;
+    wg /= nsplit;
+    const int step0 = split * a.split_steps;  // first step of this workgroup's share of the keys
+    const int kv_len = a.N - step0 * BN, nk = a.nk - step0;
     const int jq = wg % per_head;
     const int h = (wg / per_head) % a.Hq;
     const int b = wg / (per_head * a.Hq);
@@ -159,11 +167,11 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // The CAUSAL instance is the one that can hide keys: key n is visible to row m iff n <= lim(m), with
     // lim = min(m + kv_len - qo_len, kv_len - 1) under the causal flag and kv_len - 1 otherwise (a kv_len
     // that is not a multiple of 64 leaves hidden keys in the last tile).
-    const int shift = a.N - a.M;
-    const int lim = !CAUSAL ? 0 : a.causal ? min(my_m + shift, a.N - 1) : a.N - 1;                  // this lane's row
-    const int wlim = !CAUSAL ? 0 : a.causal ? min(m0 + 32 * wave + shift, a.N - 1) : a.N - 1;      // first row of the wave
+    const int shift = kv_len - a.M;
+    const int lim = !CAUSAL ? 0 : a.causal ? min(my_m + shift, kv_len - 1) : kv_len - 1;                  // this lane's row
+    const int wlim = !CAUSAL ? 0 : a.causal ? min(m0 + 32 * wave + shift, kv_len - 1) : kv_len - 1;      // first row of the wave
 
-    int nsteps = a.nk;
+    int nsteps = min(a.split_steps, nk);
     if (CAUSAL && a.causal) {
         const int last_row = min(m0 + kFastRows, a.M) - 1;
         nsteps = max(min(nsteps, (last_row + shift + BN) / BN), 0);  // 0: no row of the workgroup sees a key (qo_len > kv_len)
@@ -184,14 +192,14 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // the loop contains assembly that clobbers memory, and they are tracked by lgkmcnt, not by the vmcnt
     // the direct-to-LDS loads are tracked with
     typedef __attribute__((address_space(4))) const float* const_f32_ptr;
-    const const_f32_ptr ksp = (const_f32_ptr)(uintptr_t)(a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk);
+    const const_f32_ptr ksp = (const_f32_ptr)(uintptr_t)(a.k_scale + ((int64_t)b * a.Hkv + hk) * a.nk + step0);
     auto step_scale = [&](int j, bool hides) {  // scale of the scores of step j (hides: the step may hold hidden keys)
         float s = INT8 ? qs * ksp[j] : qs;
         if (CAUSAL && hides) s = fmaxf(s, 1.17549435e-38f);  // keeps -inf * sc = -inf for hidden keys of an all-zero K block
         return s;
     };
-    const int8_t* kg = a.k + ((int64_t)b * a.ks_b + (int64_t)hk * a.ks_h) * QB;
-    const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h;
+    const int8_t* kg = a.k + ((int64_t)b * a.ks_b + (int64_t)hk * a.ks_h + (int64_t)step0 * BN * a.ks_n) * QB;
+    const VT* vg = static_cast<const VT*>(a.v) + (int64_t)b * a.vs_b + (int64_t)hk * a.vs_h + (int64_t)step0 * BN * a.vs_n;
 
     // ---- staging: direct-to-LDS loads, 16 bytes per lane, 1 KB per wave instruction.  LDS piece
     //      p = 64 * instr + lane is chunk p % CPR of row p / CPR and receives the chunk (p % CPR) ^ swz(row)
@@ -228,10 +236,10 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     };
     // The last tile of a kv_len that is not a multiple of 64 (CAUSAL instance only): rows past the end
     // re-read the last valid row (finite values under hidden scores), through per-lane offsets of their own.
-    const bool ragged = CAUSAL && (a.N % BN) != 0;
+    const bool ragged = CAUSAL && (kv_len % BN) != 0;
     unsigned k_goff_last[F::NK], v_goff_last[F::NV];
     if (CAUSAL) {
-        const int last = (a.N - 1) % BN;
+        const int last = (kv_len - 1) % BN;
 #pragma unroll
         for (int e = 0; e < F::NK; e++) {
             const int pk = 64 * k_idx + lane, rk = pk / F::KCPR + e * (64 * kFastWaves / F::KCPR);
@@ -249,12 +257,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         constexpr int e = decltype(ec)::value;
         constexpr bool HIDES = decltype(hc)::value;  // false: the caller knows that neither tile is a ragged last one
         if constexpr (e < F::NK) {
-            const bool cut = HIDES && ragged && kt == a.nk - 1;
+            const bool cut = HIDES && ragged && kt == nk - 1;
             dma16(cut ? ktile : ktile + e * k_instr_bytes, cut ? k_goff_last[e] : k_goff,
                   lds0 + kbuf * F::K_BYTES + 1024 * (k_idx + kFastWaves * e));
         } else {
             constexpr int ev = e - F::NK;
-            const bool cut = HIDES && ragged && vt == a.nk - 1;
+            const bool cut = HIDES && ragged && vt == nk - 1;
             dma16(cut ? vtile : vtile + ev * v_instr_bytes, cut ? v_goff_last[ev] : v_goff,
                   lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
@@ -273,7 +281,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     if constexpr (MASK) {
         const int row_first = min(m0 + 32 * wave_u, a.M - 1);
         mask_row0 = static_cast<const unsigned char*>(a.mask) + (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)row_first * a.ms_m;
-        const int last_chunk = ((a.N - 1) % BN) / 16;
+        const int last_chunk = ((kv_len - 1) % BN) / 16;
 #pragma unroll
         for (int e = 0; e < 2; e++) {
             const int r = min(16 * e + (lane >> 2), a.M - 1 - row_first);
@@ -284,7 +292,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     }
     auto dma_mask = [&](int tile, int slot) {
         if constexpr (MASK) {
-            const bool cut = ragged && tile == a.nk - 1;
+            const bool cut = ragged && tile == nk - 1;
 #pragma unroll
             for (int e = 0; e < 2; e++)
                 dma16(mask_row0 + (int64_t)tile * BN, cut ? m_goff_last[e] : m_goff[e],
@@ -757,7 +765,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     int hide_from = 0;
     if (CAUSAL) {
         const int first_hidden_step = (__builtin_amdgcn_readfirstlane(wlim) + 1) / BN;  // tile that holds key wlim + 1 (may lie past the last step); wave-uniform
-        hide_from = max(min(first_hidden_step - 1, ragged ? a.nk - 4 : nsteps), 0) & ~1;
+        hide_from = max(min(first_hidden_step - 1, ragged ? nk - 4 : nsteps), 0) & ~1;
     }
     int step = 0;
     if (CAUSAL) {
@@ -778,7 +786,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const float l_o = __shfl_xor(l_i, 32);
     const float l_tot = kWholeRowSums ? l_i : half ? (l_o + l_i) : (l_i + l_o);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;  // l = 0: a row that saw no key; its output is 0, its lse -inf
-    const int64_t obase_wave = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)(m0 + 32 * wave) * a.os_n;
+    const int64_t obase_wave = (int64_t)b * a.os_b + (int64_t)h * a.os_h + (int64_t)(m0 + 32 * wave) * a.os_n + split * a.out_split_stride;
     if (a.out_dt != SAGE_F32) {
         // 16-bit outputs: a lane holds its row in 8-byte pieces, which stored directly would scatter 32
         // partial lines per instruction.  Each wave transposes its 32 rows through its own slice of LDS
@@ -823,7 +831,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             }
     }
     if (row_ok) {
-        if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m] = (__builtin_log2f(l_tot) + m_i) * a.lse_mul;
+        if (a.lse && half == 0) a.lse[((int64_t)b * a.Hq + h) * a.M + my_m + split * a.lse_split_stride] = (__builtin_log2f(l_tot) + m_i) * a.lse_mul;
     }
     __syncthreads();  // the output staging in LDS has been read: the next q-block may fill the tile buffers
   }

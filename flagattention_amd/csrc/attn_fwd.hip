@@ -466,7 +466,19 @@ int launch_mode(const AttnArgs& a, int mode, hipStream_t stream) {
 
 }  // namespace
 
-int launch_attn(const sage_attn_params& p, hipStream_t stream) {
+namespace {
+// The calls the pipelined kernel serves without a mask tensor are the ones whose keys can be split.
+int attn_key_splits(const sage_attn_params& p) {
+    if (p.mask_kind != SAGE_MASK_NONE || (p.causal && p.qo_len > p.kv_len)) return 1;
+    return attn::plan_key_split(p.batch, p.heads_q, p.qo_len, p.kv_len, p.causal != 0);
+}
+}  // namespace
+
+int64_t attn_split_workspace_bytes(const sage_attn_params& p) {
+    return attn::key_split_workspace_bytes(attn_key_splits(p), p.batch, p.heads_q, p.qo_len, p.head_dim);
+}
+
+int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     AttnArgs a{};
     a.q = (const int8_t*)p.q.ptr; a.k = (const int8_t*)p.k.ptr; a.v = p.v.ptr; a.out = p.out.ptr;
     a.q_scale = p.q_scale; a.k_scale = p.k_scale; a.lse = p.lse; a.mask = p.mask;
@@ -495,12 +507,23 @@ int launch_attn(const sage_attn_params& p, hipStream_t stream) {
         (int64_t)BN * p.v.stride_n >= (1LL << 29))
         return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: k/v sequence stride out of range for 32-bit tile offsets");
     a.total_wg = (int)total;
+    a.nsplit = 1; a.split_steps = a.nk;
     int mode = MODE_PLAIN;
     if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
     else if (additive) mode = MODE_MASK_F32;
     else if (p.causal) mode = MODE_CAUSAL;
     const bool fast = p.mask_kind == SAGE_MASK_NONE && (!p.causal || p.qo_len <= p.kv_len);
-    if (fast) return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
+    if (fast) {
+        const int nsplit = workspace ? attn_key_splits(p) : 1;
+        if (nsplit > 1 && workspace_bytes >= attn::key_split_workspace_bytes(nsplit, p.batch, p.heads_q, p.qo_len, p.head_dim)) {
+            if (total * nsplit > 0x7fffffffLL) return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: problem too large for 32-bit tile indices");
+            AttnArgs s = a;
+            attn::apply_key_split(s, nsplit, p.batch, (int)p.head_dim, workspace);
+            if (int rc = attn::launch_fast(s, (int)p.head_dim, p.v_dtype, p.causal != 0, stream)) return rc;
+            return attn::launch_split_combine(s, a, (int)p.head_dim, p.batch, stream);
+        }
+        return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
+    }
     if (p.mask_kind == SAGE_MASK_BOOL && attn::fast_serves_mask(a))
         return attn::launch_fast_masked(a, (int)p.head_dim, p.v_dtype, stream);
     if (p.head_dim == 128) {

@@ -14,7 +14,7 @@ int launch_causal(const AttnArgs& a, bool causal, hipStream_t stream) {
     AttnArgs b = a;
     const int nq2 = (a.M + kFastRows - 1) / kFastRows;
     const int per_head = a.causal ? (nq2 + 1) / 2 : nq2;  // under the causal flag a workgroup takes two q-blocks
-    b.total_wg = (int)((int64_t)a.total_wg / a.nq * per_head);
+    b.total_wg = (int)((int64_t)a.total_wg / a.nq * per_head) * a.nsplit;
     dim3 grid((unsigned)b.total_wg), block(kFastThreads);
     if (causal) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1>), grid, block, 0, stream, b, nq2);
     else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false, 1>), grid, block, 0, stream, b, nq2);

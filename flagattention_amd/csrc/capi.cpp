@@ -114,7 +114,7 @@ extern "C" int sage_k_mean_noalloc(const sage_tensor* k, int32_t k_dtype, void* 
     return launch_kmean(*k, k_dtype, km_out, out_dtype, batch, heads_kv, kv_len, head_dim, ws, (hipStream_t)stream);
 }
 
-extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
+static int check_attn_params(const sage_attn_params* p) {
     if (!p) return fail(SAGE_E_INVALID, "sage_attn_fwd: null params");
     if (!p->q.ptr || !p->k.ptr || !p->v.ptr || !p->out.ptr || !p->q_scale || !p->k_scale)
         return fail(SAGE_E_INVALID, "sage_attn_fwd: null tensor pointer");
@@ -141,14 +141,48 @@ extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
         return fail(SAGE_E_INVALID, "sage_attn_fwd: q/k/v rows must be 16-byte aligned");
     if (misaligned(p->out, dtype_bytes(p->out_dtype)))
         return fail(SAGE_E_INVALID, "sage_attn_fwd: out rows must be 16-byte aligned");
-    return launch_attn(*p, (hipStream_t)stream);
+    return SAGE_OK;
+}
+
+static int check_workspace(const char* who, const void* workspace, int64_t workspace_bytes) {
+    if (workspace_bytes < 0 || (!workspace && workspace_bytes > 0))
+        return fail(SAGE_E_INVALID, "%s: bad workspace (null with a size, or a negative size)", who);
+    if ((uintptr_t)workspace % 16 != 0) return fail(SAGE_E_INVALID, "%s: workspace must be 16-byte aligned", who);
+    return SAGE_OK;
+}
+
+extern "C" int sage_attn_fwd(const sage_attn_params* p, void* stream) {
+    if (int rc = check_attn_params(p)) return rc;
+    return launch_attn(*p, nullptr, 0, (hipStream_t)stream);
+}
+
+extern "C" int64_t sage_attn_fwd_workspace_bytes(const sage_attn_params* p) {
+    if (check_attn_params(p)) return -1;
+    return attn_split_workspace_bytes(*p);
+}
+
+extern "C" int sage_attn_fwd_ws(const sage_attn_params* p, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (int rc = check_attn_params(p)) return rc;
+    if (int rc = check_workspace("sage_attn_fwd_ws", workspace, workspace_bytes)) return rc;
+    return launch_attn(*p, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 static int check_flash_params(const sage_flash_params* p, bool forward);
 
 extern "C" int sage_flash_attn_fwd(const sage_flash_params* p, void* stream) {
     if (int rc = check_flash_params(p, true)) return rc;
-    return launch_flash_attn(*p, (hipStream_t)stream);
+    return launch_flash_attn(*p, nullptr, 0, (hipStream_t)stream);
+}
+
+extern "C" int64_t sage_flash_attn_fwd_workspace_bytes(const sage_flash_params* p) {
+    if (check_flash_params(p, true)) return -1;
+    return flash_split_workspace_bytes(*p);
+}
+
+extern "C" int sage_flash_attn_fwd_ws(const sage_flash_params* p, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (int rc = check_flash_params(p, true)) return rc;
+    if (int rc = check_workspace("sage_flash_attn_fwd_ws", workspace, workspace_bytes)) return rc;
+    return launch_flash_attn(*p, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int sage_flash_total_attention(const sage_flash_params* p, const float* log_normalizer, float* total_attention,

@@ -25,8 +25,12 @@ int launch_kmean(const sage_tensor& k, int k_dtype, void* km_out, int out_dtype,
 int launch_smooth_quant(const sage_quant_params& p, void* km_out, float* q_dot_km, void* workspace, hipStream_t stream);
 // Device address of the library's static scratch array on the current device (SAGE_K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES).
 int static_scratch(void** out);
-int launch_attn(const sage_attn_params& p, hipStream_t stream);
-int launch_flash_attn(const sage_flash_params& p, hipStream_t stream);
+// workspace: device memory for the partial results of a key split, or null (then the keys are never split);
+// *_split_workspace_bytes: what the launch would use of it (0: it would not split)
+int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+int launch_flash_attn(const sage_flash_params& p, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+int64_t attn_split_workspace_bytes(const sage_attn_params& p);
+int64_t flash_split_workspace_bytes(const sage_flash_params& p);
 int launch_flash_total_attention(const sage_flash_params& p, const float* log_normalizer, float* total, hipStream_t stream);
 
 }  // namespace sage

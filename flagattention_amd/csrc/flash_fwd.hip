@@ -16,7 +16,7 @@ int launch_dense(const AttnArgs& a, bool hides_keys, hipStream_t stream) {
     const int nq2 = (a.M + kFastRows - 1) / kFastRows;
     AttnArgs b = a;
     const int per_head = a.causal ? (nq2 + 1) / 2 : nq2;  // under the causal flag a workgroup takes two q-blocks
-    b.total_wg = (int)((int64_t)a.total_wg / nq2 * per_head);
+    b.total_wg = (int)((int64_t)a.total_wg / nq2 * per_head) * a.nsplit;
     dim3 grid((unsigned)b.total_wg), block(kFastThreads);
     if (hides_keys) hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 2>), grid, block, 0, stream, b, nq2);
     else hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, false, 2>), grid, block, 0, stream, b, nq2);
@@ -36,7 +36,15 @@ int launch_flash(const AttnArgs& a, int head_dim, int dtype, bool causal, hipStr
 
 }  // namespace attn
 
-int launch_flash_attn(const sage_flash_params& p, hipStream_t stream) {
+static int flash_key_splits(const sage_flash_params& p) {
+    return attn::plan_key_split(p.batch, p.heads_q, p.qo_len, p.kv_len, p.causal != 0);
+}
+
+int64_t flash_split_workspace_bytes(const sage_flash_params& p) {
+    return attn::key_split_workspace_bytes(flash_key_splits(p), p.batch, p.heads_q, p.qo_len, p.head_dim);
+}
+
+int launch_flash_attn(const sage_flash_params& p, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     using namespace attn;
     AttnArgs a{};
     a.q = (const int8_t*)p.q.ptr; a.k = (const int8_t*)p.k.ptr; a.v = p.v.ptr; a.out = p.out.ptr;
@@ -58,6 +66,15 @@ int launch_flash_attn(const sage_flash_params& p, hipStream_t stream) {
         (int64_t)BN * p.v.stride_n >= (1LL << 29))
         return fail(SAGE_E_UNSUPPORTED, "sage_flash_attn_fwd: k/v sequence stride out of range for 32-bit tile offsets");
     a.total_wg = (int)total;
+    a.nsplit = 1; a.split_steps = a.nk;
+    const int nsplit = workspace ? flash_key_splits(p) : 1;
+    if (nsplit > 1 && workspace_bytes >= key_split_workspace_bytes(nsplit, p.batch, p.heads_q, p.qo_len, p.head_dim)) {
+        if (total * nsplit > 0x7fffffffLL) return fail(SAGE_E_UNSUPPORTED, "sage_flash_attn_fwd: problem too large for 32-bit tile indices");
+        AttnArgs s = a;
+        apply_key_split(s, nsplit, p.batch, (int)p.head_dim, workspace);
+        if (int rc = launch_flash(s, (int)p.head_dim, p.dtype, p.causal != 0, stream)) return rc;
+        return launch_split_combine(s, a, (int)p.head_dim, p.batch, stream);
+    }
     return launch_flash(a, (int)p.head_dim, p.dtype, p.causal != 0, stream);
 }
 

@@ -79,7 +79,16 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     p.sm_scale = float(sm_scale)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        _lib.check(lib.sage_flash_attn_fwd(p, current_stream_ptr(q.device)), "sage_flash_attn_fwd")
+        # (the reference decides on its split over the keys at the same point, flash.py:73-75)
+        ws_bytes = lib.sage_flash_attn_fwd_workspace_bytes(p)
+        if ws_bytes < 0:
+            _lib.check(-1, "sage_flash_attn_fwd_workspace_bytes")
+        if ws_bytes > 0:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+            _lib.check(lib.sage_flash_attn_fwd_ws(p, ws.data_ptr(), ws_bytes, current_stream_ptr(q.device)),
+                       "sage_flash_attn_fwd_ws")
+        else:
+            _lib.check(lib.sage_flash_attn_fwd(p, current_stream_ptr(q.device)), "sage_flash_attn_fwd")
         tot = None
         if return_total_attention:
             tot = torch.empty((B, H, N), dtype=torch.float32, device=q.device)

@@ -121,6 +121,15 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
             mask_keepalive = m
             p.mask = m.data_ptr()
             p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = m.stride()
-        _lib.check(lib.sage_attn_fwd(ctypes.byref(p), current_stream_ptr(q.device)), "sage_attn_fwd")
+        # a launch with few (batch, head, q-block) items splits its keys over more workgroups, through a workspace
+        ws_bytes = lib.sage_attn_fwd_workspace_bytes(ctypes.byref(p))
+        if ws_bytes < 0:
+            _lib.check(-1, "sage_attn_fwd_workspace_bytes")
+        if ws_bytes > 0:
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+            _lib.check(lib.sage_attn_fwd_ws(ctypes.byref(p), ws.data_ptr(), ws_bytes, current_stream_ptr(q.device)),
+                       "sage_attn_fwd_ws")
+        else:
+            _lib.check(lib.sage_attn_fwd(ctypes.byref(p), current_stream_ptr(q.device)), "sage_attn_fwd")
         del mask_keepalive
     return o, lse

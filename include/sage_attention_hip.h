@@ -94,6 +94,23 @@ typedef struct sage_attn_params {
 int sage_attn_fwd(const sage_attn_params* p, void* stream);
 
 /*
+ * The same call with a workspace, for launches that would leave most of the chip idle: when
+ * batch * heads_q * ceil(qo_len / 256) is well below the 256 compute units and no mask tensor is given, the keys
+ * of every (batch, head, 256-query block) are cut into runs of whole 64-key steps, one workgroup each; the runs
+ * write normalized fp32 partial outputs and their base-2 log-sum-exps to the workspace and a second kernel
+ * combines them (out = sum_s 2^(lse_s - lse) o_s, lse = log2 sum_s 2^lse_s).  The reference's SageAttention
+ * launch has no such split (attn_qk_int8_per_block.py:176-190 is one grid over q-blocks); its dense forward does
+ * (see sage_flash_attn_fwd_ws).  Results agree with sage_attn_fwd to fp32 rounding of the combination.
+ *   sage_attn_fwd_workspace_bytes  bytes the split of this call would use; 0 = the call would not split;
+ *                                  -1 = invalid params (sage_hip_last_error says why)
+ *   workspace                      device memory, 16-byte aligned, at least that large; NULL or smaller: no split,
+ *                                  the call is sage_attn_fwd.  Contents need not be initialised and are not
+ *                                  meaningful afterwards; calls on one stream may share one workspace.
+ */
+int64_t sage_attn_fwd_workspace_bytes(const sage_attn_params* p);
+int sage_attn_fwd_ws(const sage_attn_params* p, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Mean of K over the sequence axis in a fixed fp32 order, for callers that want the library
  * to produce the `km` argument of per_block_int8 (the reference leaves km to its caller,
  * quant_per_block.py:49,53-54, so this entry point has no reference counterpart).
@@ -168,6 +185,16 @@ typedef struct sage_flash_params {
 } sage_flash_params;
 
 int sage_flash_attn_fwd(const sage_flash_params* p, void* stream);
+
+/*
+ * The dense forward with the keys split over several workgroups where the launch would otherwise leave most of
+ * the chip idle: replaces the split_kv branch of the reference's host function (src/flag_attn/flash.py:73-75,
+ * :106-141: _fwd_split_kv_kernel into fp32 partials, then _fwd_combine_kv_splits; number of runs:
+ * split_kv.py:250-278).  Workspace rules as for sage_attn_fwd_ws; the number of runs is chosen for 256 compute
+ * units with 256-query workgroups, not by the reference's formula.
+ */
+int64_t sage_flash_attn_fwd_workspace_bytes(const sage_flash_params* p);
+int sage_flash_attn_fwd_ws(const sage_flash_params* p, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Total attention of the same operator: total_attention[b, h, n] = sum over the queries m of

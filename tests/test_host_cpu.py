@@ -91,6 +91,54 @@ def test_validation_without_gpu_work():
     assert lib.sage_k_mean_workspace_bytes(2, 3, 130, 64) == 2 * 3 * 3 * 64 * 4
 
 
+def _attn_desc(batch, heads, m, n, d, causal=0, mask_kind=0):
+    from flagattention_amd import _lib
+
+    p = _lib.AttnParams()
+    for t, rows in ((p.q, m), (p.k, n), (p.v, n), (p.out, m)):
+        t.ptr, t.stride_b, t.stride_h, t.stride_n = 4096, heads * rows * d, rows * d, d
+    p.q_scale = p.k_scale = 4096
+    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = batch, heads, heads, m, n, d
+    p.v_dtype = p.out_dtype = _lib.SAGE_F16
+    p.causal, p.mask_kind = causal, mask_kind
+    if mask_kind:
+        p.mask = 4096
+    return p
+
+
+def test_key_split_plan_and_workspace_size():
+    """The split over the keys is planned on the host: which calls split, and into how much workspace."""
+    from flagattention_amd import _lib
+
+    lib = _lib.load()
+    size = lambda *a, **kw: lib.sage_attn_fwd_workspace_bytes(ctypes.byref(_attn_desc(*a, **kw)))
+    # launches that fill the 256 compute units (>= 80 % of them) or have fewer than 512 keys never split
+    assert size(4, 32, 4096, 4096, 128) == 0
+    assert size(1, 24, 32768, 32768, 128) == 0
+    assert size(1, 205, 256, 65536, 64) == 0
+    assert size(1, 4, 128, 448, 128) == 0
+    # a mask tensor keeps the call on one workgroup per q-block
+    assert size(1, 4, 128, 8192, 128, mask_kind=_lib.MASK_BOOL) == 0
+    # short queries against many keys: runs x batch x heads x rows x (head_dim + 1) fp32
+    for b, h, m, n, d in ((1, 4, 128, 8192, 128), (2, 8, 1, 4096, 64), (1, 32, 300, 32768, 128)):
+        got = size(b, h, m, n, d)
+        unit = b * h * m * (d + 1) * 4
+        assert got > 0 and got % unit == 0
+        runs = got // unit
+        nk = (n + 63) // 64
+        steps = -(-nk // runs)
+        assert 2 <= runs <= 64 and steps >= 4 and (runs - 1) * steps < nk  # every run holds a key
+        workgroups = b * h * -(-m // 256) * runs
+        assert workgroups <= 256 or runs <= 8  # (one round over the chip unless the key count is huge)
+    assert size(1, 4, 128, 8192, 128, causal=1) > 0
+    assert size(1, 4, 8192, 128, 128, causal=1) == 0  # (more queries than keys under the causal flag: general kernel)
+    bad = _attn_desc(1, 4, 128, 8192, 96)
+    assert lib.sage_attn_fwd_workspace_bytes(ctypes.byref(bad)) == -1
+    assert b"head_dim 96" in lib.sage_hip_last_error()
+    f = _lib.FlashParams()
+    assert lib.sage_flash_attn_fwd_workspace_bytes(ctypes.byref(f)) == -1
+
+
 def test_python_api_errors_on_cpu():
     from flag_attn import sage_attention as sa
 
