@@ -70,6 +70,8 @@ EXPORTS = (
     "sage_flash_attn_fwd_workspace_bytes",
     "sage_flash_attn_fwd_ws",
     "sage_flash_total_attention",
+    "sage_flash_attn_fwd_dropout",
+    "sage_flash_dropout_mask",
     "sage_k_mean",
     "sage_k_mean_workspace_bytes",
     "sage_k_mean_noalloc",
@@ -114,6 +116,12 @@ def load():
     lib.sage_flash_attn_fwd_ws.restype = ctypes.c_int
     lib.sage_flash_total_attention.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.sage_flash_total_attention.restype = ctypes.c_int
+    lib.sage_flash_attn_fwd_dropout.argtypes = [ctypes.POINTER(FlashParams), ctypes.c_float, ctypes.c_uint64,
+                                                ctypes.c_uint64, ctypes.c_void_p]
+    lib.sage_flash_attn_fwd_dropout.restype = ctypes.c_int
+    lib.sage_flash_dropout_mask.argtypes = [ctypes.c_void_p, c_i64, c_i64, c_i64, c_i64, ctypes.c_float, ctypes.c_uint64,
+                                            ctypes.c_uint64, ctypes.c_void_p]
+    lib.sage_flash_dropout_mask.restype = ctypes.c_int
     lib.sage_k_mean_workspace_bytes.argtypes = [c_i64] * 4
     lib.sage_k_mean_workspace_bytes.restype = c_i64
     lib.sage_k_mean.argtypes = [ctypes.POINTER(SageTensor), c_i32, ctypes.c_void_p, c_i32, c_i64, c_i64, c_i64,

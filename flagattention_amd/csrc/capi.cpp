@@ -185,6 +185,35 @@ extern "C" int sage_flash_attn_fwd_ws(const sage_flash_params* p, void* workspac
     return launch_flash_attn(*p, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+// dropout_p in (0, 1); the element index of the random stream is 32-bit arithmetic in the reference
+static int check_dropout(const char* who, float dropout_p, int64_t batch, int64_t heads, int64_t qo_len, int64_t kv_len,
+                         uint64_t offset) {
+    if (!(dropout_p > 0.0f && dropout_p < 1.0f)) return fail(SAGE_E_INVALID, "%s: dropout_p must lie in (0, 1)", who);
+    if (batch <= 0 || heads <= 0 || qo_len <= 0 || kv_len <= 0) return fail(SAGE_E_INVALID, "%s: sizes must be positive", who);
+    const int64_t lim = 1LL << 31;
+    if (batch >= lim || heads >= lim || qo_len >= lim || kv_len >= lim || batch * heads >= lim ||
+        batch * heads * qo_len >= lim || batch * heads * qo_len * kv_len >= lim)
+        return fail(SAGE_E_UNSUPPORTED, "%s: batch x heads x qo_len x kv_len must stay below 2^31 (the 32-bit element "
+                    "index of the random stream wraps beyond)", who);
+    if (offset >= (1ULL << 63)) return fail(SAGE_E_INVALID, "%s: offset must be below 2^63", who);
+    return SAGE_OK;
+}
+
+extern "C" int sage_flash_attn_fwd_dropout(const sage_flash_params* p, float dropout_p, uint64_t seed, uint64_t offset,
+                                           void* stream) {
+    if (int rc = check_flash_params(p, true)) return rc;
+    if (int rc = check_dropout("sage_flash_attn_fwd_dropout", dropout_p, p->batch, p->heads_q, p->qo_len, p->kv_len, offset))
+        return rc;
+    return launch_flash_dropout(*p, dropout_p, seed, offset, (hipStream_t)stream);
+}
+
+extern "C" int sage_flash_dropout_mask(uint8_t* mask, int64_t batch, int64_t heads_q, int64_t qo_len, int64_t kv_len,
+                                       float dropout_p, uint64_t seed, uint64_t offset, void* stream) {
+    if (!mask) return fail(SAGE_E_INVALID, "sage_flash_dropout_mask: null mask");
+    if (int rc = check_dropout("sage_flash_dropout_mask", dropout_p, batch, heads_q, qo_len, kv_len, offset)) return rc;
+    return launch_dropout_mask(mask, batch * heads_q * qo_len * kv_len, dropout_p, seed, offset, (hipStream_t)stream);
+}
+
 extern "C" int sage_flash_total_attention(const sage_flash_params* p, const float* log_normalizer, float* total_attention,
                                           void* stream) {
     if (int rc = check_flash_params(p, false)) return rc;

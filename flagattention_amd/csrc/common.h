@@ -32,5 +32,7 @@ int launch_flash_attn(const sage_flash_params& p, void* workspace, int64_t works
 int64_t attn_split_workspace_bytes(const sage_attn_params& p);
 int64_t flash_split_workspace_bytes(const sage_flash_params& p);
 int launch_flash_total_attention(const sage_flash_params& p, const float* log_normalizer, float* total, hipStream_t stream);
+int launch_flash_dropout(const sage_flash_params& p, float dropout_p, uint64_t seed, uint64_t offset, hipStream_t stream);
+int launch_dropout_mask(uint8_t* mask, int64_t count, float dropout_p, uint64_t seed, uint64_t offset, hipStream_t stream);
 
 }  // namespace sage

@@ -197,6 +197,23 @@ int64_t sage_flash_attn_fwd_workspace_bytes(const sage_flash_params* p);
 int sage_flash_attn_fwd_ws(const sage_flash_params* p, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * The dense forward with dropout on P (src/flag_attn/flash.py:66-71 host side, :387-391, :467-502 kernel branch
+ * IS_DROPOUT): element (b, h, m, n) of P survives iff
+ *     rand(seed, offset + ((b * heads_q + h) * qo_len + m) * kv_len + n) > dropout_p
+ * with Triton's tl.rand of six rounds (Philox-4x32 on the two words of the 64-bit offset, key = the two words of
+ * the seed, first output word -> fp32 in [0, 1)); the softmax row sums and the log normalizer do not see the mask,
+ * the output is scaled by 1 / (1 - dropout_p).  seed and offset are the caller's (the reference takes them from
+ * torch's CUDA generator, dropout.py:17-28).  dropout_p in (0, 1); batch * heads_q * qo_len * kv_len < 2^31.
+ * A plain kernel, an order of magnitude slower than sage_flash_attn_fwd: the generator dominates.
+ *
+ * sage_flash_dropout_mask writes the same mask on its own (src/flag_attn/testing/dropout.py:19-39):
+ *   mask   [batch, heads_q, qo_len, kv_len] bytes, contiguous, 1 = kept
+ */
+int sage_flash_attn_fwd_dropout(const sage_flash_params* p, float dropout_p, uint64_t seed, uint64_t offset, void* stream);
+int sage_flash_dropout_mask(uint8_t* mask, int64_t batch, int64_t heads_q, int64_t qo_len, int64_t kv_len,
+                            float dropout_p, uint64_t seed, uint64_t offset, void* stream);
+
+/*
  * Total attention of the same operator: total_attention[b, h, n] = sum over the queries m of
  * softmax(sm_scale * Q K^T [+ causal])[m, n], recomputed from Q, K and the log normalizer that
  * sage_flash_attn_fwd returned for the same arguments (src/flag_attn/total.py:22-160, called from

@@ -15,7 +15,9 @@ non-causal case and for causal with M == N; for M != N and for rows that see no 
 against a brute-force loop over (query, key) pairs on tiny inputs; the log normalizer against
 ``log(sum(exp(.)))`` computed in float64; the total attention against the same brute-force loop
 (sum over the queries of exp(score - log normalizer)) and against two invariants: it sums to the number of
-queries that see a key, and with V = identity the output's column sums are the total attention.
+queries that see a key, and with V = identity the output's column sums are the total attention.  The dropout
+branch: with V = identity the output IS the masked P / (1 - p), checked element by element against the brute-force
+P; an all-True mask with p = 0 changes nothing.
 """
 from __future__ import annotations
 
@@ -24,10 +26,13 @@ import math
 import torch
 
 
-def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False, upcast=True, return_total_attention=False):
+def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False, upcast=True, return_total_attention=False,
+              dropout_p=0.0, dropout_mask=None):
     """q [B,H,M,D], k/v [B,Hk,N,D] (CPU).  Returns o (input dtype), or (o, log_normalizer fp32 [B,H,M]), or with
     return_total_attention (o, log_normalizer or None, total_attention fp32 [B,H,N]): the column sums of P over
-    the queries (testing/flash.py:66-67)."""
+    the queries (testing/flash.py:66-67).  dropout_mask (bool [B,H,M,N], True = kept) zeroes elements of the
+    normalized P, and P V is scaled by 1 / (1 - dropout_p) (testing/flash.py:69-74); the log normalizer and the
+    total attention are those of the undropped P."""
     input_dtype = q.dtype
     if upcast:
         q, k, v = q.float(), k.float(), v.float()
@@ -49,9 +54,12 @@ def attention(q, k, v, causal=False, sm_scale=None, return_log_normalizer=False,
     p = torch.softmax(scores, dim=-1, dtype=torch.float32)
     if causal:
         p = torch.where(visible, p, 0.0)  # also turns the NaN rows of queries that see no key into zeros
-    o = (p.to(v.dtype) @ v).to(input_dtype)
+    total = p.sum(dim=-2) if return_total_attention else None
+    if dropout_mask is not None:
+        p = p.masked_fill(~dropout_mask, 0.0)
+    o = ((p.to(v.dtype) @ v) * (1.0 / (1 - dropout_p))).to(input_dtype)
     if return_total_attention:
-        return o, log_normalizer, p.sum(dim=-2)
+        return o, log_normalizer, total
     return (o, log_normalizer) if return_log_normalizer else o
 
 

@@ -7,6 +7,7 @@
 * K mean: agreement with the fp32 mean to one 16-bit ulp and an exact case.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -323,3 +324,101 @@ def test_flash_oracle_total_attention(causal, m, n):
     eye = torch.eye(n).expand(2, 2, n, n).contiguous()  # V = identity: o[m, :] = P[m, :]
     o_eye, _, tot_eye = FO.attention(q, k, eye, causal=causal, sm_scale=0.6, return_total_attention=True)
     torch.testing.assert_close(o_eye.sum(dim=-2), tot_eye, atol=1e-5, rtol=1e-5)
+
+
+# ---- dropout: the random stream and the masked closed form
+
+_PHILOX_KAT = [
+    # Random123 kat_vectors, ten rounds: (width, counter, key, output)
+    (32, (0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+    (32, (0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+    (32, (0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+     (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
+    (64, (0, 0, 0, 0), (0, 0), (0x16554d9eca36314c, 0xdb20fe9d672d0fdc, 0xd7e772cee186176b, 0x7e68b68aec7ba23b)),
+    (64, (0xffffffffffffffff,) * 4, (0xffffffffffffffff,) * 2,
+     (0x87b092c3013fe90b, 0x438c3c67be8d0224, 0x9cc7d7c69cd777b6, 0xa09caebf594f0ba0)),
+    (64, (0x243f6a8885a308d3, 0x13198a2e03707344, 0xa4093822299f31d0, 0x082efa98ec4e6c89),
+     (0x452821e638d01377, 0xbe5466cf34e90c6c),
+     (0xa528f45403e61d95, 0x38c72dbd566e9788, 0xa5a1610e72fd18b5, 0x57bd43b5e52b7fe6)),
+]
+
+
+@pytest.mark.parametrize("width,counter,key,expected", _PHILOX_KAT)
+def test_philox_known_answers(width, counter, key, expected):
+    """The published known-answer vectors of Philox-4x32-10 and Philox-4x64-10: a swapped multiplier, a key that is
+    bumped before instead of after the round, or high/low words taken the wrong way round fails all of them."""
+    from oracle import philox_oracle as P
+
+    got = tuple(int(x[0]) for x in P.philox(counter, key, width, 10))
+    assert got == expected
+
+
+def test_uniform_conversion_ends_of_the_range():
+    """Signed reading of the word, negative values folded by -x - 1, times 4.6566127342e-10 in fp32: 0 and -1 give
+    0, the two words next to the sign change give the largest value, which stays below 1."""
+    from oracle import philox_oracle as P
+
+    u = P.uniform(np.array([0, 0xFFFFFFFF, 0x7FFFFFFF, 0x80000000, 0x40000000, 0xBFFFFFFF], dtype=np.uint64))
+    assert u.dtype == np.float32
+    assert u[0] == 0 and u[1] == 0
+    assert u[2] == u[3] == np.float32(2147483647.0) * np.float32(4.6566127342e-10) and u[2] < 1
+    assert u[4] == u[5] == np.float32(0x40000000) * np.float32(4.6566127342e-10) and abs(float(u[4]) - 0.5) < 1e-6
+
+
+def test_dropout_mask_matches_reference_golden():
+    """Masks written by the reference's own helper kernel under Triton's CPU interpreter (six rounds, key words from
+    the seed, counter words from the 64-bit offset, `> dropout_p`): offsets on both sides of 2^31 and beyond 2^32,
+    seeds with high bits, a row longer than the helper's 1024-column run."""
+    from oracle import philox_oracle as P
+
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "dropout_golden.npz"))
+    assert len(g["names"]) >= 6
+    for name in g["names"]:
+        B, H, M, N, seed, offset = (int(x) for x in g[f"{name}.args"])
+        mask = P.keep_mask(B, H, M, N, float(g[f"{name}.p"]), seed, offset)
+        assert np.array_equal(mask, g[f"{name}.mask"]), name
+
+
+@pytest.mark.parametrize("p", [0.1, 0.5, 0.8])
+def test_dropout_mask_keeps_the_right_fraction(p):
+    from oracle import philox_oracle as P
+
+    mask = P.keep_mask(2, 3, 64, 500, p, 987654321, 1 << 20)
+    assert abs(mask.mean() - (1 - p)) < 4 * math.sqrt(p * (1 - p) / mask.size)
+    # another offset is the same stream shifted, not a fresh one
+    shifted = P.keep_mask(2, 3, 64, 500, p, 987654321, (1 << 20) + 500)
+    assert np.array_equal(shifted.reshape(-1)[:-500], mask.reshape(-1)[500:])
+    with pytest.raises(ValueError):
+        P.keep_mask(1 << 10, 1 << 10, 1 << 6, 1 << 5, p, 1, 0)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_oracle_dropout_branch(causal):
+    """With V = identity the output is the masked, rescaled P itself: every element is checked against the
+    brute-force P; the log normalizer and the total attention do not see the mask; an all-True mask with p = 0 is
+    the plain call.  A mask applied before the normalization or a missing 1 / (1 - p) fails."""
+    from oracle import flash_oracle as FO
+
+    g = torch.Generator().manual_seed(5)
+    m, n, p = 6, 9, 0.4
+    q = torch.randn(1, 2, m, 8, generator=g)
+    k = torch.randn(1, 2, n, 8, generator=g)
+    eye = torch.eye(n).expand(1, 2, n, n).contiguous()
+    keep = torch.rand(1, 2, m, n, generator=g) > p
+    o, lse, tot = FO.attention(q, k, eye, causal=causal, sm_scale=0.5, return_log_normalizer=True,
+                               return_total_attention=True, dropout_p=p, dropout_mask=keep)
+    _, blse = _brute_force_attention(q, k, torch.zeros(1, 2, n, 8), causal, 0.5)
+    for h in range(2):
+        for mm in range(m):
+            for nn in range(n):
+                visible = not causal or nn <= mm + (n - m)
+                want = 0.0
+                if visible and bool(keep[0, h, mm, nn]):
+                    want = math.exp(0.5 * float(q[0, h, mm].double() @ k[0, h, nn].double()) - float(blse[0, h, mm])) / (1 - p)
+                assert abs(float(o[0, h, mm, nn]) - want) < 1e-5
+    plain, plain_lse, plain_tot = FO.attention(q, k, eye, causal=causal, sm_scale=0.5, return_log_normalizer=True,
+                                               return_total_attention=True)
+    torch.testing.assert_close(lse, plain_lse)
+    torch.testing.assert_close(tot, plain_tot)
+    same = FO.attention(q, k, eye, causal=causal, sm_scale=0.5, dropout_p=0.0, dropout_mask=torch.ones_like(keep))
+    torch.testing.assert_close(same, plain)
