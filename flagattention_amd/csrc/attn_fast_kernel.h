@@ -131,9 +131,12 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 
 
     // workgroup -> (batch, head, q-block); consecutive logical ids stay on one XCD (8 XCDs, round robin)
-    // Under the causal flag a workgroup takes two q-blocks of its head, one after the other: block
-    // nq2 - 1 - j (long rows) and block j (short rows), so that every workgroup of the launch runs about
-    // the same number of steps (one q-block alone runs between 1/nq2 and all of them).
+    // Under the causal flag a workgroup takes two q-blocks of its head, one after the other: block j (short
+    // rows) and block nq2 - 1 - j (long rows), so that every workgroup of the launch runs about the same number
+    // of steps (one q-block alone runs between 1/nq2 and all of them).  Short block first: the workgroups of a
+    // head then start their long walks over the keys 4 steps apart, a window of tiles that stays in the XCD's L2;
+    // with the long block first the short ones re-read the head's first tiles after they had been evicted
+    // (1.35x the K/V bytes from memory at 8192 keys).
     int wg = blockIdx.x;
     if ((a.total_wg & 7) == 0) wg = (wg & 7) * (a.total_wg >> 3) + (wg >> 3);
     const bool paired = CAUSAL && a.causal;
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const int lane = tid & 63;
     const int l32 = lane & 31;
     const int half = lane >> 5;
-    const int iq = paired && pass == 0 ? nq2 - 1 - jq : jq;
+    const int iq = paired && pass == 1 ? nq2 - 1 - jq : jq;
     const int m0 = iq * kFastRows;
     const int my_m = m0 + 32 * wave + l32;
     const bool row_ok = my_m < a.M;

@@ -110,8 +110,6 @@ def test_unbuilt_features_raise(gpu_device):
 
     q, k, v = (t.to(gpu_device) for t in _inputs(6, 1, 2, 2, 64, 64, 64, torch.float16))
     with pytest.raises(NotImplementedError):
-        flag_attn.flash_attention(q, k, v, dropout_p=0.1)
-    with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q[..., :48], k[..., :48], v[..., :48])
     with pytest.raises(NotImplementedError):
         flag_attn.flash_attention(q.requires_grad_(), k, v)
