@@ -147,3 +147,73 @@ def test_flash_forward_with_split_keys(B, Hq, Hk, M, N, D, causal, dtype, gpu_de
     inf = torch.isinf(L_ref)
     assert torch.equal(torch.isinf(L.cpu()), inf)
     torch.testing.assert_close(L.cpu()[~inf], L_ref[~inf], atol=2e-3, rtol=2e-4)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_sage_split_layouts_output_types_grouped_heads(layout, out_dtype, gpu_device):
+    """The combine kernel writes through the caller's strides and in the caller's type; heads share K/V runs."""
+    from flagattention_amd import _lib
+    from flag_attn import sage_attention as sa
+
+    g = torch.Generator().manual_seed(24)
+    b, hq, hkv, m, n, d = 2, 6, 2, 200, 1500, 128
+    q = torch.randn(b, hq, m, d, generator=g).to(torch.float16)
+    k = torch.randn(b, hkv, n, d, generator=g).to(torch.float16)
+    v = torch.randn(b, hkv, n, d, generator=g).to(torch.float16)
+    if layout == "NHD":
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    q8, qs, k8, ks = O.per_block_int8(q, k, tensor_layout=layout)
+    args = [t.to(gpu_device) for t in (q8, k8, v, qs, ks)]
+    for return_lse in (True, False):
+        o, lse = sa.sage_attention(*args, tensor_layout=layout, output_dtype=out_dtype, return_lse=return_lse)
+        torch.cuda.synchronize()
+        assert o.dtype == out_dtype and o.shape == q8.shape
+        expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, layout)
+        cos, _, max_abs = O.accuracy_metrics(o.float().cpu(), expected)
+        assert cos >= 0.9995 and max_abs <= 2e-2
+        if return_lse:
+            torch.testing.assert_close(lse.cpu(), expected_lse, atol=2e-3, rtol=1e-4)
+        else:
+            assert lse.numel() == 0 and lse.device.type == "cpu"
+    p = _lib.AttnParams()  # (the shape does split)
+    from flagattention_amd.sage_attention.attention import DTYPE_CODE, tensor_desc
+    p.q, p.k, p.v, p.out = (tensor_desc(t, layout == "HND") for t in (args[0], args[1], args[2], o))
+    p.q_scale, p.k_scale = args[3].data_ptr(), args[4].data_ptr()
+    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = b, hq, hkv, m, n, d
+    p.v_dtype, p.out_dtype = DTYPE_CODE[torch.float16], DTYPE_CODE[out_dtype]
+    assert _lib.load().sage_attn_fwd_workspace_bytes(ctypes.byref(p)) > 0
+
+
+def test_split_launch_in_a_captured_graph(gpu_device):
+    """Both kernels of a split launch only enqueue work on the caller's stream: a captured graph (workspace from the
+    capture's memory pool) replays to the eager result, with eager work between the replays."""
+    from flag_attn import sage_attention as sa
+
+    q8, qs, k8, ks, v = (t.to(gpu_device) for t in _sage_inputs(25, 1, 4, 4, 128, 2048, 128, torch.bfloat16))
+
+    def run(x):
+        return sa.sage_attention(x, k8, v, qs, ks, output_dtype=torch.bfloat16, return_lse=True)
+
+    want = [t.clone() for t in run(q8)]
+    flipped = q8.flip(2).contiguous()
+    want_flipped = [t.clone() for t in run(flipped)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    static_q = q8.clone()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(static_q)  # warm-up on the capture stream (allocator)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = run(static_q)
+    for rep in range(4):
+        expect = want_flipped if rep % 2 else want
+        static_q.copy_(flipped if rep % 2 else q8)
+        run(q8.roll(1, 2))  # eager work in between, through the same allocator
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(captured, expect):
+            assert torch.equal(a, b), f"replay {rep}"
