@@ -4,7 +4,6 @@ Gate (north star): cosine >= 0.9995 and max-abs <= 2e-2 against the dequantized 
 same int8 inputs; the reference's own test tolerance atol = rtol = 2e-2 on output and LSE
 (tests/flag_attn/test_sage_attention.py:104-105,156-157) is asserted too.
 """
-import math
 
 import pytest
 import torch
