@@ -25,8 +25,9 @@ __device__ __forceinline__ uint32_t philox6_first_word(uint32_t c0, uint32_t c1,
     uint32_t c2 = 0, c3 = 0;
 #pragma unroll
     for (int r = 0; r < 6; r++) {
-        const uint32_t hi_b = __umulhi(ROUND_B, c2), lo_b = ROUND_B * c2;
-        const uint32_t hi_a = __umulhi(ROUND_A, c0), lo_a = ROUND_A * c0;
+        const uint64_t pb = (uint64_t)ROUND_B * c2, pa = (uint64_t)ROUND_A * c0;
+        const uint32_t hi_b = (uint32_t)(pb >> 32), lo_b = (uint32_t)pb;
+        const uint32_t hi_a = (uint32_t)(pa >> 32), lo_a = (uint32_t)pa;
         c0 = hi_b ^ c1 ^ k0;
         c2 = hi_a ^ c3 ^ k1;
         c1 = lo_b;
