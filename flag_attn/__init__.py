@@ -6,5 +6,6 @@ package.  Metadata strings follow the reference's src/flag_attn/__init__.py:22-2
 """
 from flagattention_amd import backend_info, device, flash_attention, vendor, vendor_name
 from . import sage_attention  # noqa: F401  (stays a namespace, as in the reference :115-117)
+from . import testing  # noqa: F401
 
-__all__ = ["sage_attention", "flash_attention", "device", "vendor", "vendor_name", "backend_info"]
+__all__ = ["sage_attention", "flash_attention", "testing", "device", "vendor", "vendor_name", "backend_info"]

@@ -72,8 +72,8 @@ def _inputs(seed, B, H, Hk, M, N, D, dtype, order, std=1.0):
 ])
 def test_forward_with_dropout_against_reference_rule(B, H, Hk, M, N, D, causal, dropout_p, dtype, order, gpu_device):
     import flag_attn
-    from flagattention_amd.flash import recompute_mask
 
+    recompute_mask = flag_attn.testing.recompute_mask  # (the name the reference's own test calls, :327)
     q, k, v = _inputs(31, B, H, Hk, M, N, D, dtype, order)
     torch.manual_seed(1000 * M + N)
     o, L, tot, seed, offset = flag_attn.flash_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), causal,
