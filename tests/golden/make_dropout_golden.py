@@ -28,6 +28,7 @@ CASES = [
     ("counter_crosses_2_31", 1, 2, 4, 33, 0.5, 7, (1 << 31) - 100),  # int32 counter wraps to negative values
     ("offset_above_2_31", 1, 2, 4, 33, 0.5, 7, (1 << 31) + 4),       # an int64 kernel argument
     ("large_offset", 2, 2, 3, 17, 0.9, (1 << 40) + 99, (1 << 40) + 12),
+    ("carry_into_high_word", 1, 1, 3, 40, 0.5, 11, (1 << 32) - 50),  # the low counter word wraps inside the mask
 ]
 
 

@@ -372,7 +372,7 @@ def test_dropout_mask_matches_reference_golden():
     from oracle import philox_oracle as P
 
     g = np.load(os.path.join(os.path.dirname(__file__), "golden", "dropout_golden.npz"))
-    assert len(g["names"]) >= 6
+    assert len(g["names"]) >= 7
     for name in g["names"]:
         B, H, M, N, seed, offset = (int(x) for x in g[f"{name}.args"])
         mask = P.keep_mask(B, H, M, N, float(g[f"{name}.p"]), seed, offset)
