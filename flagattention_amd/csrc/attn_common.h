@@ -40,6 +40,8 @@ struct AttnArgs {
     int32_t total_wg;
     int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
     int32_t mask_dt;   // storage type of an additive mask (SAGE_F32 / SAGE_F16 / SAGE_BF16)
+    int32_t mask_padded;  // bool mask rows are readable, and zero, up to the next multiple of 16 bytes past kv_len
+    int32_t mask_causal;  // the bool mask is False wherever n > m + (kv_len - qo_len): tiles beyond need no visit
     // Split of the keys over several workgroups per (batch, head, q-block) (never under a mask tensor): workgroup s
     // of `nsplit` takes steps s * split_steps .. and writes an fp32 partial output and its base-2 log-sum-exp to
     // out + s * out_split_stride / lse + s * lse_split_stride, which a second kernel combines.  Unsplit: 1, nk, 0, 0.

@@ -105,14 +105,16 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 // QB = 1: int8 Q and K with per-block scales (SageAttention).  QB = 2: Q and K in V's 16-bit type, one
 // scale for the whole call (dense attention); in bytes a 16-bit K row of head_dim D is laid out, loaded
 // and read exactly like an int8 row of head_dim 2 D.
-// MASK: a bool mask tensor [B, Hq, M, N] (bytes 0 / 1, rows 16-byte aligned, kv_len a multiple of 16) on top of
+// MASK: a bool mask tensor [B, Hq, M, N] (bytes 0 / 1, rows 16-byte aligned and readable, as zeros, up to the next
+// multiple of 16 keys: kv_len a multiple of 16, or rows the caller padded) on top of
 // the key-hiding instance.  Every wave stages the 32 x 64 mask bytes of its own rows and step in a private slice
 // of LDS (direct-to-LDS loads, three steps resident) and multiplies P by them.  The reference's arithmetic for
 // rows that have not seen a visible key yet (scores of hidden keys are s - 1e6, not -inf:
 // attn_qk_int8_per_block.py:46-52) and its skipping of 128 x 64 tiles without a visible key (:33-36) are
 // served by the path that redoes a step: such rows start from the reference point -inf, which drives every
-// step into that path until the row has seen a key.  Additive masks and masks with unaligned rows stay with the
-// general kernel (attn_fwd.hip).
+// step into that path until the row has seen a key.  a.mask_causal: the caller folded the causal mask into the
+// tensor, so tiles beyond the causal limit of the workgroup's last row need no visit.  Additive masks and masks
+// with unaligned rows stay with the general kernel (attn_fwd.hip).
 constexpr int kMaskSlots = 3;                       // steps of mask bytes resident per wave
 constexpr int kMaskWaveBytes = 32 * BN;            // 32 rows x 64 keys x 1 byte
 constexpr int kMaskBytes = kMaskSlots * kFastWaves * kMaskWaveBytes;
@@ -163,7 +165,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const int lane = tid & 63;
     const int l32 = lane & 31;
     const int half = lane >> 5;
-    const int iq = paired && pass == 1 ? nq2 - 1 - jq : jq;
+    // (a mask with the causal mask folded in: no pairs, the q-blocks with the most tiles are handed out first)
+    const int iq = (paired && pass == 1) || (MASK && a.mask_causal) ? nq2 - 1 - jq : jq;
     const int m0 = iq * kFastRows;
     const int my_m = m0 + 32 * wave + l32;
     const bool row_ok = my_m < a.M;
@@ -175,7 +178,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     const int wlim = !CAUSAL ? 0 : a.causal ? min(m0 + 32 * wave + shift, kv_len - 1) : kv_len - 1;      // first row of the wave
 
     int nsteps = min(a.split_steps, nk);
-    if (CAUSAL && a.causal) {
+    if (CAUSAL && (a.causal || (MASK && a.mask_causal))) {  // (a mask with the causal mask folded in: same bound)
         const int last_row = min(m0 + kFastRows, a.M) - 1;
         nsteps = max(min(nsteps, (last_row + shift + BN) / BN), 0);  // 0: no row of the workgroup sees a key (qo_len > kv_len)
     }
@@ -450,7 +453,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
     if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
     dma_mask(0, 0);
-    dma_mask(min(1, nsteps - 1), 1);
+    dma_mask(max(min(1, nsteps - 1), 0), 1);  // (nsteps = 0: a workgroup that sees no key; tile 0 exists all the same)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);

@@ -492,11 +492,15 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
     a.groups = (int)(p.heads_q / p.heads_kv);
     a.out_dt = p.out_dtype; a.causal = p.causal ? 1 : 0;
     a.lse_mul = 1.0f;
+    const bool is_bool = p.mask_kind == SAGE_MASK_BOOL || p.mask_kind == SAGE_MASK_BOOL_PADDED ||
+                         p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL;
+    a.mask_padded = p.mask_kind == SAGE_MASK_BOOL_PADDED || p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL;
+    a.mask_causal = p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL;
     const bool additive = p.mask_kind == SAGE_MASK_F32 || p.mask_kind == SAGE_MASK_F16 || p.mask_kind == SAGE_MASK_BF16;
     a.mask_dt = p.mask_kind == SAGE_MASK_F16 ? SAGE_F16 : p.mask_kind == SAGE_MASK_BF16 ? SAGE_BF16 : SAGE_F32;
     if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_n == 1) {
         // runs of four entries are read with one load where they are naturally aligned
-        const int64_t esz = p.mask_kind == SAGE_MASK_BOOL ? 1 : dtype_bytes(a.mask_dt), align = 4 * esz;
+        const int64_t esz = is_bool ? 1 : dtype_bytes(a.mask_dt), align = 4 * esz;
         a.mask_vec = ((uintptr_t)p.mask % align) == 0 && (p.mask_stride_b * esz) % align == 0 &&
                      (p.mask_stride_h * esz) % align == 0 && (p.mask_stride_m * esz) % align == 0;
     }
@@ -509,7 +513,7 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
     a.total_wg = (int)total;
     a.nsplit = 1; a.split_steps = a.nk;
     int mode = MODE_PLAIN;
-    if (p.mask_kind == SAGE_MASK_BOOL) mode = MODE_MASK_BOOL;
+    if (is_bool) mode = MODE_MASK_BOOL;
     else if (additive) mode = MODE_MASK_F32;
     else if (p.causal) mode = MODE_CAUSAL;
     const bool fast = p.mask_kind == SAGE_MASK_NONE && (!p.causal || p.qo_len <= p.kv_len);
@@ -524,7 +528,7 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
         }
         return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
     }
-    if (p.mask_kind == SAGE_MASK_BOOL && attn::fast_serves_mask(a))
+    if (is_bool && attn::fast_serves_mask(a))
         return attn::launch_fast_masked(a, (int)p.head_dim, p.v_dtype, stream);
     if (p.head_dim == 128) {
         return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)

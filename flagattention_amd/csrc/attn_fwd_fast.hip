@@ -1,6 +1,6 @@
 // SageAttention forward for gfx950, pipelined kernel: the int8 Q, K instances of attn_fast_kernel.h.
 // They serve every call without a mask tensor (causal only with qo_len <= kv_len; any kv_len) and bool mask tensors
-// with 16-byte aligned rows, under the
+// with 16-byte aligned rows (padded by the caller where kv_len is not a multiple of 16), under the
 // arithmetic contract of FlagAttention src/flag_attn/sage_attention/attn_qk_int8_per_block.py:20-127
 // (per-block scales, base-2 online softmax, lse = log2(l) + m).
 #include "attn_fast_kernel.h"
@@ -34,10 +34,12 @@ int launch_masked(const AttnArgs& a, hipStream_t stream) {
 }  // namespace
 
 // A bool mask tensor the pipelined kernel can stage with 16-byte loads: contiguous along the keys, every row start
-// 16-byte aligned, kv_len a multiple of 16 (so that no load reaches past the end of a row), no causal flag on top.
+// 16-byte aligned, no load that reaches past the end of a row (kv_len a multiple of 16, or rows that the caller
+// padded with zeros to one), no causal flag on top.
 bool fast_serves_mask(const AttnArgs& a) {
     return a.mask != nullptr && !a.causal && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 && a.ms_b % 16 == 0 &&
-           a.ms_h % 16 == 0 && a.ms_m % 16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 26) && a.N % 16 == 0;
+           a.ms_h % 16 == 0 && a.ms_m % 16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 26) &&
+           (a.N % 16 == 0 || a.mask_padded);
 }
 
 int launch_fast_masked(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream) {

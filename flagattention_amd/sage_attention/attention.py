@@ -14,6 +14,41 @@ from ._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, 
 
 BLOCK_M = 128  # attn_qk_int8_per_block.py:131
 BLOCK_N = 64  # attn_qk_int8_per_block.py:132
+_STAGED_MASK_MAX_BYTES = 1 << 31  # largest staging copy of a bool mask this wrapper makes
+
+
+def _bool_mask_is_direct(m: torch.Tensor, kv_len: int) -> bool:
+    """Can the pipelined kernel stage this (already expanded) bool mask as it is?  16-byte loads along the keys:
+    unit stride, 16-byte aligned rows, and no load that passes the end of a row."""
+    return (m.stride(-1) == 1 and m.data_ptr() % 16 == 0 and all(s % 16 == 0 for s in m.stride()[:-1])
+            and m.stride(2) < (1 << 26) and kv_len % 16 == 0)
+
+
+def stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=None):
+    """A copy of a bool mask (or of the causal mask alone, ``mask=None``) that the pipelined kernel can stage: rows
+    padded with False to a multiple of 16 keys, unit stride along the keys, broadcast dimensions kept as they are;
+    under ``causal`` the bottom-right aligned causal mask ``n <= m + (N - M)`` is folded in (one bool mask that is
+    the conjunction of the two is what the reference's mask path would be given).  Returns the ``[b, h, M, N]``
+    view to pass as SAGE_MASK_BOOL_PADDED, or None when the copy would pass ``_STAGED_MASK_MAX_BYTES``."""
+    padded = (kv_len + 15) // 16 * 16
+    if mask is None:
+        bb, hh, mm = 1, 1, qo_len
+    else:
+        m4 = mask.reshape((1,) * (4 - mask.dim()) + tuple(mask.shape))
+        bb, hh, mm = m4.shape[0], m4.shape[1], (qo_len if causal else m4.shape[2])
+        device = mask.device
+    if bb * hh * mm * padded > _STAGED_MASK_MAX_BYTES:
+        return None
+    buf = torch.zeros((bb, hh, mm, padded), dtype=torch.bool, device=device)
+    live = buf[..., :kv_len]
+    if mask is not None:
+        live.copy_(m4.expand(bb, hh, mm, kv_len))
+    else:
+        live.fill_(True)
+    if causal:
+        rows = torch.arange(qo_len, device=buf.device).unsqueeze(1) + (kv_len - qo_len)
+        live.logical_and_(torch.arange(kv_len, device=buf.device).unsqueeze(0) <= rows)
+    return live.expand(b, h, qo_len, kv_len)
 
 
 def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
@@ -106,6 +141,23 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
         mask_keepalive = None
         if attn_mask is not None:
             require_gpu(attn_mask, "attn_mask")
+        staged = None
+        if attn_mask is not None and attn_mask.dtype == torch.bool:
+            # bool masks run on the pipelined kernel; one that it cannot stage as it is (rows that are not 16-byte
+            # aligned, kv_len not a multiple of 16, a causal flag on top) goes there through a padded copy
+            if causal or not _bool_mask_is_direct(attn_mask.expand(b, h_qo, qo_len, kv_len), kv_len):
+                staged = stage_bool_mask(attn_mask, b, h_qo, qo_len, kv_len, causal)
+        elif attn_mask is None and causal and qo_len > kv_len:
+            # rows that see no key follow the reference's mask arithmetic (-1e6, whole-tile skip), which the
+            # pipelined kernel implements for mask tensors: hand it the causal mask as one
+            staged = stage_bool_mask(None, b, h_qo, qo_len, kv_len, True, device=q.device)
+        if staged is not None:
+            p.causal = 0
+            p.mask_kind = _lib.MASK_BOOL_PADDED_CAUSAL if causal else _lib.MASK_BOOL_PADDED
+            mask_keepalive = staged
+            p.mask = staged.data_ptr()
+            p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = staged.stride()
+        elif attn_mask is not None:
             m = attn_mask
             if m.dtype == torch.bool:
                 p.mask_kind = _lib.MASK_BOOL

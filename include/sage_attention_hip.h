@@ -23,7 +23,8 @@ extern "C" {
 #endif
 
 enum sage_dtype { SAGE_F16 = 0, SAGE_BF16 = 1, SAGE_F32 = 2 };
-enum sage_mask_kind { SAGE_MASK_NONE = 0, SAGE_MASK_BOOL = 1, SAGE_MASK_F32 = 2, SAGE_MASK_F16 = 3, SAGE_MASK_BF16 = 4 };
+enum sage_mask_kind { SAGE_MASK_NONE = 0, SAGE_MASK_BOOL = 1, SAGE_MASK_F32 = 2, SAGE_MASK_F16 = 3, SAGE_MASK_BF16 = 4,
+                      SAGE_MASK_BOOL_PADDED = 5, SAGE_MASK_BOOL_PADDED_CAUSAL = 6 };
 enum sage_status {
     SAGE_OK = 0,
     SAGE_E_INVALID = -1,     /* bad argument (shape, dtype, stride, null pointer) */
@@ -75,6 +76,13 @@ int sage_per_block_int8(const sage_quant_params* p, void* stream);
  *   lse          optional [B, Hq, M] fp32 contiguous, base-2 log-sum-exp (:124-127); NULL = none
  *   mask         optional [B, Hq, M, N] through 4 strides (elements, 0 = broadcast);
  *                SAGE_MASK_BOOL: 1 byte per element, 1 = keep, 0 = hide (:33-36,48); other byte values are not allowed;
+ *                SAGE_MASK_BOOL_PADDED: the same, and the caller guarantees that every mask row can be read up to the
+ *                next multiple of 16 bytes past kv_len and holds zeros there (a staging copy with padded rows): with
+ *                16-byte aligned rows such a mask runs on the pipelined kernel for any kv_len, where a plain
+ *                SAGE_MASK_BOOL needs kv_len % 16 == 0 for that;
+ *                SAGE_MASK_BOOL_PADDED_CAUSAL: a padded mask of which the caller also guarantees mask[m, n] = 0 for
+ *                n > m + (kv_len - qo_len) (the causal mask is folded in): the pipelined kernel then does not visit
+ *                the key tiles beyond that limit, which the reference would skip one by one as all-False tiles;
  *                SAGE_MASK_F32 / SAGE_MASK_F16 / SAGE_MASK_BF16: additive, in that storage type (:38,50)
  *   causal       non-zero adds the bottom-right aligned causal mask n <= m + (N - M), handled
  *                like a bool mask (tiles that are entirely masked are skipped)

@@ -280,6 +280,95 @@ def test_bool_masks_with_aligned_rows(kind, d, vdtype, m, n, gpu_device):
     torch.testing.assert_close(lse.cpu()[hidden], expected_lse[hidden], atol=1.0, rtol=1e-5)
 
 
+def _check_masked(o, lse, expected, expected_lse, what):
+    assert bool(torch.isfinite(o).all())
+    if float(expected.abs().max()) == 0.0:  # no query sees a key: every tile skipped, zero rows
+        assert float(o.abs().max()) == 0.0, what
+    else:
+        _gate(o, expected, what)
+    normal = expected_lse > -1.0e5  # rows that saw a key; the others: -inf (every tile skipped) or about -1e6
+    assert torch.equal(torch.isneginf(lse.cpu()), torch.isneginf(expected_lse))
+    torch.testing.assert_close(lse.cpu()[normal], expected_lse[normal], atol=6e-3, rtol=1e-4)
+    hidden = ~normal & torch.isfinite(expected_lse)
+    torch.testing.assert_close(lse.cpu()[hidden], expected_lse[hidden], atol=1.0, rtol=1e-5)
+
+
+@pytest.mark.parametrize("kind", ["random", "broadcast", "window", "holes"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n", [(300, 500), (129, 70), (600, 1001), (200, 257), (700, 333)])
+def test_bool_masks_of_any_length_and_with_the_causal_flag(kind, causal, m, n, gpu_device):
+    """kv_len that is not a multiple of 16, and the causal flag on top of a mask: the host stages a copy with padded
+    rows (and the causal mask folded in) for the pipelined kernel.  Same oracle, same -1e6 / tile-skip semantics;
+    more queries than keys under the causal flag leaves rows without any visible key."""
+    b, hq, hkv = 2, 4, 2
+    q8, qs, k8, ks, v = _quantized(45, b, hq, hkv, m, n, 128, torch.bfloat16)
+    mask = _mask_case(kind, b, hq, m, n, 11)
+    o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask.to(gpu_device), causal=causal, return_lse=True,
+                  output_dtype=torch.float32)
+    both = mask & (torch.arange(n)[None, :] <= torch.arange(m)[:, None] + (n - m)) if causal else mask
+    expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, attn_mask=both)
+    _check_masked(o, lse, expected, expected_lse, f"{kind} causal={causal}")
+
+
+def test_mask_views_with_odd_strides(gpu_device):
+    """Masks the kernel cannot read as they are: transposed storage, a column slice of a wider mask (rows that are
+    not 16-byte aligned, bytes of other columns behind every row), a key-padding mask [B, 1, 1, N]."""
+    b, hq, hkv, m, n = 2, 4, 2, 260, 330
+    q8, qs, k8, ks, v = _quantized(46, b, hq, hkv, m, n, 64, torch.float16)
+    g = torch.Generator().manual_seed(12)
+    wide = (torch.rand(b, hq, m, n + 37, generator=g) > 0.3).to(gpu_device)
+    transposed = (torch.rand(b, hq, n, m, generator=g) > 0.3).to(gpu_device).transpose(2, 3)
+    padding = torch.ones(b, 1, 1, n, dtype=torch.bool)
+    padding[0, ..., 200:] = False
+    padding[1, ..., 321:] = False
+    for name, mask in (("slice", wide[..., 5:5 + n]), ("transposed", transposed), ("key padding", padding.to(gpu_device))):
+        o, lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask, return_lse=True, output_dtype=torch.float32)
+        expected, expected_lse = C.attention_blockwise(q8, k8, v, qs, ks, attn_mask=mask.cpu().expand(b, hq, m, n))
+        _check_masked(o, lse, expected, expected_lse, name)
+
+
+@pytest.mark.parametrize("n", [70, 257, 512])
+def test_bool_mask_kinds_through_the_c_abi(n, gpu_device):
+    """SAGE_MASK_BOOL on rows that are not 16-byte aligned stays on the general kernel; the same mask as
+    SAGE_MASK_BOOL_PADDED (rows padded with zeros to a multiple of 16) takes the pipelined one.  Both against the
+    oracle, and against each other."""
+    import ctypes
+
+    from flagattention_amd import _lib
+    from flagattention_amd.sage_attention._common import DTYPE_CODE, tensor_desc
+
+    b, h, m, d = 1, 2, 200, 128
+    q8, qs, k8, ks, v = (t.to(gpu_device) for t in _quantized(47, b, h, h, m, n, d, torch.bfloat16))
+    mask = _mask_case("holes", b, h, m, n, 13)
+    expected, expected_lse = C.attention_blockwise(q8.cpu(), k8.cpu(), v.cpu(), qs.cpu(), ks.cpu(), attn_mask=mask)
+    lib = _lib.load()
+    outs = []
+    for kind in (_lib.MASK_BOOL, _lib.MASK_BOOL_PADDED):
+        if kind == _lib.MASK_BOOL:  # rows start at odd addresses
+            store = torch.zeros(b, h, m, n + 3, dtype=torch.bool, device=gpu_device)
+            view = store[..., 1:1 + n]
+        else:
+            store = torch.zeros(b, h, m, (n + 15) // 16 * 16, dtype=torch.bool, device=gpu_device)
+            view = store[..., :n]
+        view.copy_(mask)
+        o = torch.empty(q8.shape, dtype=torch.float32, device=gpu_device)
+        lse = torch.empty(b, h, m, dtype=torch.float32, device=gpu_device)
+        p = _lib.AttnParams()
+        p.q, p.k, p.v, p.out = (tensor_desc(t, True) for t in (q8, k8, v, o))
+        p.q_scale, p.k_scale, p.lse = qs.data_ptr(), ks.data_ptr(), lse.data_ptr()
+        p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = b, h, h, m, n, d
+        p.v_dtype, p.out_dtype = DTYPE_CODE[torch.bfloat16], DTYPE_CODE[torch.float32]
+        p.mask_kind, p.mask = kind, view.data_ptr()
+        p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = view.stride()
+        assert lib.sage_attn_fwd(ctypes.byref(p), torch.cuda.current_stream().cuda_stream) == 0, lib.sage_hip_last_error()
+        torch.cuda.synchronize()
+        _check_masked(o, lse, expected, expected_lse, f"kind {kind}")
+        outs.append(o)
+    torch.testing.assert_close(outs[0], outs[1], atol=5e-3, rtol=1e-2)
+    p.mask_kind = 7
+    assert lib.sage_attn_fwd(ctypes.byref(p), None) == -1 and b"mask_kind" in lib.sage_hip_last_error()
+
+
 @pytest.mark.parametrize("pattern", sorted(_SCALE_PATTERNS))
 def test_bool_mask_with_row_maximum_that_moves(pattern, gpu_device):
     m, n = 320, 768

@@ -139,6 +139,37 @@ def test_key_split_plan_and_workspace_size():
     assert lib.sage_flash_attn_fwd_workspace_bytes(ctypes.byref(f)) == -1
 
 
+def test_bool_mask_staging_copy():
+    """The copy of a bool mask that the host hands to the pipelined kernel: same values, broadcast dimensions kept,
+    rows padded with False to a multiple of 16 keys and 16-byte aligned, the causal mask folded in on request."""
+    import torch
+
+    from flagattention_amd.sage_attention.attention import _bool_mask_is_direct, stage_bool_mask
+
+    g = torch.Generator().manual_seed(0)
+    for shape, causal, (b, h, m, n) in [((1, 1, 5, 37), False, (2, 3, 5, 37)), ((2, 1, 1, 70), False, (2, 3, 9, 70)),
+                                        ((2, 3, 9, 70), True, (2, 3, 9, 70)), ((9, 70), True, (2, 3, 9, 70)),
+                                        ((1, 1, 12, 7), True, (1, 2, 12, 7)), ((3, 1, 64), False, (2, 3, 1, 64))]:
+        mask = torch.rand(shape, generator=g) > 0.4
+        staged = stage_bool_mask(mask, b, h, m, n, causal)
+        want = mask.expand(b, h, m, n)
+        if causal:
+            want = want & (torch.arange(n)[None, :] <= torch.arange(m)[:, None] + (n - m))
+        assert staged.shape == (b, h, m, n) and torch.equal(staged, want)
+        assert staged.stride(-1) == 1 and all(x % 16 == 0 for x in staged.stride()[:-1]) and staged.data_ptr() % 16 == 0
+        row = (n + 15) // 16 * 16
+        whole = staged.as_strided((staged.untyped_storage().nbytes() // row, row), (row, 1))
+        assert not bool(whole[:, n:].any())  # the padding of every stored row is False
+        for dim, size in enumerate(mask.reshape((1,) * (4 - mask.dim()) + tuple(mask.shape)).shape[:2]):
+            if size == 1 and (b, h)[dim] > 1:
+                assert staged.stride(dim) == 0  # broadcast over batch / heads stays a broadcast
+    only_causal = stage_bool_mask(None, 1, 2, 12, 7, True, device="cpu")
+    assert torch.equal(only_causal[0, 1], torch.arange(7)[None, :] <= torch.arange(12)[:, None] - 5)
+    aligned = torch.ones(2, 3, 8, 64, dtype=torch.bool)
+    assert _bool_mask_is_direct(aligned, 64) and not _bool_mask_is_direct(aligned[..., :60], 60)
+    assert not _bool_mask_is_direct(aligned.transpose(2, 3), 8)
+
+
 def test_python_api_errors_on_cpu():
     from flag_attn import sage_attention as sa
 
