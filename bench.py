@@ -132,16 +132,27 @@ def main_flash(args):
     q, k, v = ((t.transpose(1, 2) if layout == "NHD" else t) for t in (q0, k0, v0))
     qd, kd, vd = ((t.to(dev).transpose(1, 2) if layout == "NHD" else t.to(dev)) for t in (q0, k0, v0))
 
+    drop = args.dropout
+    if drop and b * h * n * n >= 2 ** 31:
+        print("bench.py: --dropout needs batch * heads * seq_len^2 < 2^31 (the reference's 32-bit element index)", file=sys.stderr)
+        sys.exit(2)
+
     def step():
-        return flag_attn.flash_attention(qd, kd, vd, causal)
+        return flag_attn.flash_attention(qd, kd, vd, causal, dropout_p=drop)
 
     o = step()
     torch.cuda.synchronize()
     parity = None
     if n <= 8192:  # one (batch, head) against the CPU oracle, under the reference's acceptance rule
         sl = (slice(0, 1), slice(0, 1))
-        ref = FO.attention(q[sl], k[sl], v[sl], causal, upcast=True)
-        yard = FO.max_diff(FO.attention(q[sl], k[sl], v[sl], causal, upcast=False), ref)
+        keep = None
+        if drop:  # the mask of that call, rebuilt on the CPU from its seed and offset
+            from oracle import philox_oracle as PO
+            o, _, _, seed, offset = flag_attn.flash_attention(qd, kd, vd, causal, dropout_p=drop, return_seed_offset=True)
+            torch.cuda.synchronize()
+            keep = torch.from_numpy(PO.keep_mask(1, 1, n, n, drop, seed, offset))  # (batch 0, head 0: the first M*N draws)
+        ref = FO.attention(q[sl], k[sl], v[sl], causal, upcast=True, dropout_p=drop, dropout_mask=keep)
+        yard = FO.max_diff(FO.attention(q[sl], k[sl], v[sl], causal, upcast=False, dropout_p=drop, dropout_mask=keep), ref)
         got = FO.max_diff(o[sl].cpu(), ref)
         parity = {"max_diff": got, "max_diff_of_16bit_closed_form": yard, "within_reference_rule": got <= 2 * yard + 1e-5,
                   "checked_on": "batch 0, head 0 vs the CPU oracle"}
@@ -175,10 +186,11 @@ def main_flash(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "clock_ramp_steps": ramp_steps,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if dtype == torch.bfloat16 else "f16", "data": "synthetic (seed 42, generated on CPU, copied to HBM before timing)",
-        "config": {"workload": "flash_attention_" + desc.split("_smoothk")[0], "batch": b, "heads": h, "seq_len": n, "head_dim": d,
-                   "layout": layout, "causal": causal},
+        "config": {"workload": "flash_attention_" + desc.split("_smoothk")[0] + (f"_dropout{drop}" if drop else ""), "batch": b,
+                   "heads": h, "seq_len": n, "head_dim": d, "layout": layout, "causal": causal, "dropout_p": drop},
         "parity": parity,
-        "roofline": {"kernel": "sage_attn_fwd_fast_kernel (16-bit Q, K instance)", "bound": "mfma",
+        "roofline": {"kernel": "flash_dropout_fwd_kernel (bound by the integer multiplier, priced against MFMA all the same)" if drop
+                     else "sage_attn_fwd_fast_kernel (16-bit Q, K instance)", "bound": "mfma",
                      "achieved": round(ops / (avg * 1e-3) / 1e12, 2), "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": measured_traffic_bytes(name, "flash_attention"),
                      "algorithmic_bytes_per_launch": 4 * numel * 2, "algorithmic_ops_per_launch": ops,
@@ -198,6 +210,10 @@ def main():
     ap.add_argument("--op", default="sage_attention", choices=["sage_attention", "flash_attention"],
                     help="sage_attention (default): K mean + quantization + INT8-QK forward; flash_attention: the dense 16-bit forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--mask", default="none", choices=["none", "bool"],
+                    help="side path of --op sage_attention: forward under a seeded [1, 1, M, N] bool mask (30 %% hidden)")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="side path of --op flash_attention: dropout probability of the forward call")
     ap.add_argument("--min-warmup-seconds", type=float, default=0.15,
                     help="the warm-up is stretched to at least this much load before the sustained timing (clock ramp)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -225,6 +241,10 @@ def main():
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     smooth = name != "c4"
     out_dtype = dtype
+    mask_cpu = mask_dev = None
+    if args.mask == "bool":
+        mask_cpu = torch.rand(1, 1, n, n, generator=torch.Generator().manual_seed(43)) > 0.3
+        mask_dev = mask_cpu.to(dev)
 
     def step(ev=None):
         if ev:
@@ -232,7 +252,7 @@ def main():
         q8, qs, k8, ks = sa.per_block_int8(qd, kd, tensor_layout=layout, smooth_k=smooth)
         if ev:
             ev[1].record()
-        o, _ = sa.sage_attention(q8, k8, vd, qs, ks, tensor_layout=layout, output_dtype=out_dtype, causal=causal)
+        o, _ = sa.sage_attention(q8, k8, vd, qs, ks, tensor_layout=layout, attn_mask=mask_dev, output_dtype=out_dtype, causal=causal)
         if ev:
             ev[2].record()
         return q8, qs, k8, ks, o
@@ -253,7 +273,7 @@ def main():
     scale_exact = bool(torch.equal(got[1], want[1]) and torch.equal(got[3], want[3]))
     cos = max_abs = None
     if n <= 8192:
-        ref, _ = O.attention_dequant(got[0][:, :1], got[2][:, :1], cut(v, 1), got[1][:, :1], got[3][:, :1], causal=causal)
+        ref, _ = O.attention_dequant(got[0][:, :1], got[2][:, :1], cut(v, 1), got[1][:, :1], got[3][:, :1], attn_mask=mask_cpu, causal=causal)
         cos, _, max_abs = O.accuracy_metrics(cut(o, 1).float(), ref)
 
     # ---- timed region: W warm-up steps, then exactly K steps.  The GPU clock needs about 0.1 s of load to
@@ -322,8 +342,9 @@ def main():
         "dtype": "int8 QK^T (int32 acc) + bf16 PV (fp32 acc), fp32 softmax" if dtype == torch.bfloat16
         else "int8 QK^T (int32 acc) + fp16 PV (fp32 acc), fp32 softmax",
         "data": "synthetic (seed 42, N(0,1) generated on CPU, copied to HBM before timing)",
-        "config": {"workload": desc, "batch": b, "heads": h, "seq_len": n, "head_dim": d, "layout": layout,
-                   "causal": causal, "smooth_k": smooth, "blkq": 128, "blkk": 64},
+        "config": {"workload": desc + ("_boolmask" if mask_dev is not None else ""), "batch": b, "heads": h, "seq_len": n,
+                   "head_dim": d, "layout": layout, "causal": causal, "smooth_k": smooth, "blkq": 128, "blkk": 64,
+                   "attn_mask": "[1, 1, M, N] bool, 30 % hidden, seed 43" if mask_dev is not None else None},
         "pct_of_mixed_mfma_peak": round(100 * value / PEAK_MIXED_TOPS, 2),
         "attention_only": {
             "us_per_call_avg": round(attn_avg * 1e3, 1),
@@ -346,7 +367,7 @@ def main():
             "peak": round(PEAK_MIXED_TOPS, 1),
             "unit": "TFLOP/s",
             "frac": round(attn_tops / PEAK_MIXED_TOPS, 4),
-            "traffic": measured_traffic_bytes(name),
+            "traffic": measured_traffic_bytes(name) if mask_dev is None else None,
             "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, read from profiles/attention_hbm_traffic.txt)",
             "algorithmic_bytes_per_launch": numel * (1 + 1 + esz) + numel * out_dtype.itemsize,
             "peak_note": "mixed dense-MFMA roofline: half the ops INT8 at 5000 TOP/s, half 16-bit at 2500 TFLOP/s",
