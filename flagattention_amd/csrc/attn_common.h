@@ -42,6 +42,10 @@ struct AttnArgs {
     int32_t mask_dt;   // storage type of an additive mask (SAGE_F32 / SAGE_F16 / SAGE_BF16)
     int32_t mask_padded;  // bool mask rows are readable, and zero, up to the next multiple of 16 bytes past kv_len
     int32_t mask_causal;  // the bool mask is False wherever n > m + (kv_len - qo_len): tiles beyond need no visit
+    // Heads that take turns within one q-block in the order of the workgroups (1: a head's q-blocks follow each
+    // other).  Under a mask shared by the heads, head_tile heads x several q-blocks run side by side on an XCD, so
+    // that both the mask tiles (shared by the heads) and the K/V tiles (shared by the q-blocks) are re-read from L2.
+    int32_t head_tile;
     // Split of the keys over several workgroups per (batch, head, q-block) (never under a mask tensor): workgroup s
     // of `nsplit` takes steps s * split_steps .. and writes an fp32 partial output and its base-2 log-sum-exp to
     // out + s * out_split_stride / lse + s * lse_split_stride, which a second kernel combines.  Unsplit: 1, nk, 0, 0.

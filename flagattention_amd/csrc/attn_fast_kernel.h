@@ -151,8 +151,11 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     wg /= nsplit;
     const int step0 = split * a.split_steps;  // first step of this workgroup's share of the keys
     const int kv_len = a.N - step0 * BN, nk = a.nk - step0;
-    const int jq = wg % per_head;
-    const int h = (wg / per_head) % a.Hq;
+    // heads that alternate within a q-block: measured to pay only under a mask with the causal mask folded in
+    // (-7 %; +1..3 % for other shared masks, whose launches keep a head's q-blocks together for its K/V)
+    const int ht = MASK && a.mask_causal ? a.head_tile : 1;
+    const int jq = (wg / ht) % per_head;
+    const int h = (wg / (ht * per_head)) % (a.Hq / ht) * ht + wg % ht;
     const int b = wg / (per_head * a.Hq);
     const int hk = h / a.groups;
   for (int pass = 0; pass < 2; pass++) {

@@ -93,9 +93,10 @@ __global__ __launch_bounds__(kThreads, 2) void sage_attn_fwd_kernel(AttnArgs a) 
         const int per_xcd = a.total_wg >> 3;
         if ((a.total_wg & 7) == 0) wg = (wg & 7) * per_xcd + (wg >> 3);
     }
-    int iq = wg % a.nq;
+    const int ht = MODE >= MODE_MASK_BOOL ? a.head_tile : 1;  // heads that alternate within a q-block (shared mask)
+    int iq = (wg / ht) % a.nq;
     if (MODE == MODE_CAUSAL) iq = a.nq - 1 - iq;  // longest rows first
-    const int h = (wg / a.nq) % a.Hq;
+    const int h = (wg / (ht * a.nq)) % (a.Hq / ht) * ht + wg % ht;
     const int b = wg / (a.nq * a.Hq);
     const int hk = h / a.groups;
     const int m0 = iq * BM;
@@ -512,6 +513,9 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
         return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: k/v sequence stride out of range for 32-bit tile offsets");
     a.total_wg = (int)total;
     a.nsplit = 1; a.split_steps = a.nk;
+    a.head_tile = 1;
+    if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_h == 0 && p.heads_q > 1)
+        a.head_tile = p.heads_q % 8 == 0 ? 8 : p.heads_q % 4 == 0 ? 4 : p.heads_q % 2 == 0 ? 2 : 1;
     int mode = MODE_PLAIN;
     if (is_bool) mode = MODE_MASK_BOOL;
     else if (additive) mode = MODE_MASK_F32;
