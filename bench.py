@@ -40,16 +40,83 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attention_hbm_traffic.txt")
 
 
+KERNEL_SOURCES = ("attn_fast_kernel.h", "attn_common.h", "attn_fwd_fast.hip", "flash_fwd.hip")
+
+
+def kernel_sources_sha():
+    """Short hash of the sources of the pipelined attention kernel: a traffic figure counts only for the build it
+    was measured on."""
+    import hashlib
+
+    hsh = hashlib.sha256()
+    for f in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "flagattention_amd", "csrc", f), "rb") as fh:
+            hsh.update(fh.read())
+    return hsh.hexdigest()[:12]
+
+
 def measured_traffic_bytes(name, op="sage_attention"):
+    """(bytes per launch, hash of the kernel sources the line was measured on) or (None, None).  A line measured on
+    other kernel sources than the tree's gives (None, that hash): the caller reports traffic null."""
     try:
         with open(TRAFFIC_FILE) as f:
             for line in f:
                 parts = line.split()
                 if len(parts) >= 3 and parts[0] == op and parts[1] == name:
-                    return float(parts[2])
+                    sha = next((x.split("=", 1)[1] for x in parts if x.startswith("kernel_sha=")), None)
+                    try:
+                        current = kernel_sources_sha()
+                    except OSError:
+                        current = None
+                    if sha is not None and sha == current:
+                        return float(parts[2]), sha
+                    return None, sha
     except OSError:
         pass
-    return None
+    return None, None
+
+
+class ClockSampler:
+    """Samples the shader clock (the active level of /sys/class/drm/card*/device/pp_dpm_sclk) from a thread while a
+    timed region runs.  No file, no samples: mean() is None."""
+
+    def __init__(self, period_s=0.002):
+        import glob
+        import threading
+
+        self.files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.samples, self.period, self._stop = [], period_s, False
+        self.thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        import re
+
+        while not self._stop:
+            for f in self.files:
+                try:
+                    with open(f) as fh:
+                        for ln in fh:
+                            if "*" in ln:
+                                mt = re.search(r"(\d+)\s*mhz", ln, re.I)
+                                if mt:
+                                    self.samples.append(int(mt.group(1)))
+                except OSError:
+                    pass
+            time.sleep(self.period)
+
+    def __enter__(self):
+        if self.files:
+            self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self.files:
+            self.thread.join()
+        return False
+
+    def mean(self):
+        return sum(self.samples) / len(self.samples) if self.samples else None
 
 
 WORKLOADS = {
@@ -107,7 +174,7 @@ def cpu_baseline(name, q, k, v, budget_s=12.0):
     t = sorted(times)[len(times) // 2]
     return {
         "value": per_head_ops * heads / t / 1e12,
-        "unit": "TOPS (effective, same op count)",
+        "unit": "TOPS (effective, same op count; extrapolated from the sampled (batch, head) slices to the full call)",
         "cores": torch.get_num_threads(),
         "host_cpu_count": os.cpu_count(),
         "kind": "port",
@@ -192,7 +259,7 @@ def main_flash(args):
         "roofline": {"kernel": "flash_dropout_fwd_kernel (bound by the integer multiplier, priced against MFMA all the same)" if drop
                      else "sage_attn_fwd_fast_kernel (16-bit Q, K instance)", "bound": "mfma",
                      "achieved": round(ops / (avg * 1e-3) / 1e12, 2), "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": measured_traffic_bytes(name, "flash_attention"),
+                     "frac": round(ops / (avg * 1e-3) / 1e12 / PEAK_16BIT_TFLOPS, 4), "traffic": measured_traffic_bytes(name, "flash_attention")[0],
                      "algorithmic_bytes_per_launch": 4 * numel * 2, "algorithmic_ops_per_launch": ops,
                      "avg_launch_ms": round(avg, 4)},
     }
@@ -303,7 +370,9 @@ def main():
             step()
         torch.cuda.synchronize()
         ramp_steps += 10
-    wall, events = timed(args.steps)
+    with ClockSampler() as clock:
+        wall, events = timed(args.steps)
+    sclk = clock.mean()
     # (c) cold: one step after a second of idleness, no warm-up at all
     time.sleep(1.0)
     wall_cold, ev_cold = timed(1)
@@ -320,6 +389,9 @@ def main():
     quant_bytes = (esz + 1) * 2 * numel + (esz * numel if smooth else 0)  # Q,K read+write (+ K read by the mean)
     value = ops / (ms_per_step * 1e-3) / 1e12
     attn_tops = ops / (attn_avg * 1e-3) / 1e12
+    traffic, traffic_sha = measured_traffic_bytes(name) if mask_dev is None else (None, None)
+    asked_attn_ms = sum(e[1].elapsed_time(e[2]) for e in ev_asked) / len(ev_asked)
+    NOMINAL_MHZ = 2400.0  # the clock the published peaks are quoted at
     result = {
         "metric": f"effective TOPS + % of dense MFMA peak, B{b} H{h} N{n} D{d} {'bf16' if dtype == torch.bfloat16 else 'fp16'}; us/call",
         "value": round(value, 2),
@@ -331,7 +403,9 @@ def main():
                        "as_requested: K steps right after the W warm-up steps asked for, from an idle GPU; cold: one step after 1 s idle",
         "as_requested": {"ms_per_step": round(wall_asked / args.steps * 1e3, 4),
                          "value": round(ops_of_step / (wall_asked / args.steps) / 1e12, 2),
-                         "attention_us_avg": round(sum(e[1].elapsed_time(e[2]) for e in ev_asked) / len(ev_asked) * 1e3, 1)},
+                         "attention_us_avg": round(asked_attn_ms * 1e3, 1),
+                         "frac_whole_step": round(ops_of_step / (wall_asked / args.steps) / 1e12 / PEAK_MIXED_TOPS, 4),
+                         "frac_attention": round(ops / (asked_attn_ms * 1e-3) / 1e12 / PEAK_MIXED_TOPS, 4)},
         "cold": {"ms_per_step": round(wall_cold * 1e3, 4), "value": round(ops_of_step / wall_cold / 1e12, 2),
                  "attention_us": round(ev_cold[0][1].elapsed_time(ev_cold[0][2]) * 1e3, 1)},
         "ms_per_step": round(ms_per_step, 4),
@@ -367,8 +441,16 @@ def main():
             "peak": round(PEAK_MIXED_TOPS, 1),
             "unit": "TFLOP/s",
             "frac": round(attn_tops / PEAK_MIXED_TOPS, 4),
-            "traffic": measured_traffic_bytes(name) if mask_dev is None else None,
-            "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, read from profiles/attention_hbm_traffic.txt)",
+            "frac_whole_step": round(value / PEAK_MIXED_TOPS, 4),
+            "sclk_mhz_mean": None if sclk is None else round(sclk, 0),
+            "sclk_samples": len(clock.samples),
+            "frac_at_measured_clock": None if sclk is None else round(attn_tops / (PEAK_MIXED_TOPS * sclk / NOMINAL_MHZ), 4),
+            "clock_note": "peak is quoted at %d MHz; frac_at_measured_clock prices the same launch time against the peak "
+                          "scaled to the shader clock sampled (pp_dpm_sclk) during the timed region" % NOMINAL_MHZ,
+            "traffic": traffic,
+            "traffic_kernel_sha": traffic_sha,
+            "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, read from profiles/attention_hbm_traffic.txt; "
+                            "null when that line was measured on other kernel sources than this tree's: kernel_sha)",
             "algorithmic_bytes_per_launch": numel * (1 + 1 + esz) + numel * out_dtype.itemsize,
             "peak_note": "mixed dense-MFMA roofline: half the ops INT8 at 5000 TOP/s, half 16-bit at 2500 TFLOP/s",
             "algorithmic_ops_per_launch": ops,
@@ -379,6 +461,31 @@ def main():
                            "frac": round(quant_bytes / (quant_med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                            "algorithmic_bytes_per_step": quant_bytes},
     }
+    if name == "c1":
+        # host-side cost per call at the reference's own test shape, where the kernels take a few microseconds: wall
+        # time of N back-to-back calls (the launch loop is what bounds it) beside the GPU time of the same calls
+        def host_cost(fn, ncalls=1000):
+            for _ in range(100):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            for _ in range(ncalls):
+                fn()
+            e1.record()
+            t_issue = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            return {"host_us_per_call": round(t_issue / ncalls * 1e6, 2), "gpu_span_us_per_call": round(e0.elapsed_time(e1) / ncalls * 1e3, 2),
+                    "calls": ncalls}
+
+        km_c1 = sa.k_mean(kd, layout)
+        result["host_cost"] = {
+            "per_block_int8": host_cost(lambda: sa.per_block_int8(qd, kd, km=km_c1, tensor_layout=layout)),
+            "forward": host_cost(lambda: sa.sage_attention(q8, k8, vd, qs, ks, tensor_layout=layout, output_dtype=out_dtype)),
+            "note": "host_us_per_call: wall time to issue one call from Python (argument checks, output allocation, one "
+                    "C-ABI call), N calls back to back; gpu_span_us_per_call: first-to-last GPU time of the same N calls / N",
+        }
     if args.calibration_copy_mib > 0:
         src = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -105,7 +105,7 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 // QB = 1: int8 Q and K with per-block scales (SageAttention).  QB = 2: Q and K in V's 16-bit type, one
 // scale for the whole call (dense attention); in bytes a 16-bit K row of head_dim D is laid out, loaded
 // and read exactly like an int8 row of head_dim 2 D.
-// MASK: a bool mask tensor [B, Hq, M, N] (bytes 0 / 1, rows 16-byte aligned and readable, as zeros, up to the next
+// MASK: a bool mask tensor [B, Hq, M, N] (a byte per entry, non-zero = visible; rows 16-byte aligned and readable, as zeros, up to the next
 // multiple of 16 keys: kv_len a multiple of 16, or rows the caller padded) on top of
 // the key-hiding instance.  Every wave stages the 32 x 64 mask bytes of its own rows and step in a private slice
 // of LDS (direct-to-LDS loads, three steps resident) and multiplies P by them.  The reference's arithmetic for
@@ -547,12 +547,14 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
             float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
             if constexpr (MASK) {
-                // P of a hidden key is 0 (mask bytes are 0 / 1).  An overflowed P times 0 is NaN: the row sum then
+                // P of a hidden key is 0.  An overflowed P times 0 is NaN: the row sum then
                 // sends the step into the path that redoes it.
                 if constexpr (w == 0 && tp < 3) mask_words(mslot, tp + 1, mw[(tp + 1) & 1][0], mw[(tp + 1) & 1][1]);
+                // (any non-zero byte keeps the key: the conversion clamps to [0, 1], an output modifier of the same
+                // instruction)
                 const unsigned word = mw[tp & 1][w >> 1];
-                p0 *= (float)((word >> (16 * (w & 1))) & 0xffu);
-                p1 *= (float)((word >> (16 * (w & 1) + 8)) & 0xffu);
+                p0 *= __builtin_amdgcn_fmed3f((float)((word >> (16 * (w & 1))) & 0xffu), 0.0f, 1.0f);
+                p1 *= __builtin_amdgcn_fmed3f((float)((word >> (16 * (w & 1) + 8)) & 0xffu), 0.0f, 1.0f);
             }
             pf[tp][2 * w] = (VT)p0;
             pf[tp][2 * w + 1] = (VT)p1;

@@ -10,11 +10,15 @@ import ctypes
 import torch
 
 from .. import _lib
-from ._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, tensor_desc
+from ._common import (DTYPE_CODE, current_stream_ptr, device_guard, plans, require_gpu, rows_aligned,
+                      split_workspace, tensor_desc)
 
 BLOCK_M = 128  # attn_qk_int8_per_block.py:131
 BLOCK_N = 64  # attn_qk_int8_per_block.py:132
-_STAGED_MASK_MAX_BYTES = 1 << 31  # largest staging copy of a bool mask this wrapper makes
+# Largest staging copy of a bool mask this wrapper makes.  A mask that needs a larger one (a per-head [B, H, M, N]
+# mask with unaligned rows at long sequences) is served by the general kernel as it is, without a copy.
+_STAGED_MASK_MAX_BYTES = 256 << 20
+_STAGED = {}  # device index -> (key, StagedBoolMask): the mask staged last on that device
 
 
 def _bool_mask_is_direct(m: torch.Tensor, kv_len: int) -> bool:
@@ -24,16 +28,38 @@ def _bool_mask_is_direct(m: torch.Tensor, kv_len: int) -> bool:
             and m.stride(2) < (1 << 26) and kv_len % 16 == 0)
 
 
+class StagedBoolMask:
+    """A bool mask in the form the pipelined kernel stages from (what ``stage_bool_mask`` returns).  Pass it as
+    ``attn_mask`` to ``forward`` / ``sage_attention`` with the same ``causal`` flag: the call then uses it as it is.
+    ``tensor`` is the ``[b, h, M, N]`` view (rows padded with False to a multiple of 16 keys in memory); the
+    source mask may be freed or changed afterwards."""
+
+    __slots__ = ("tensor", "b", "h", "qo_len", "kv_len", "causal")
+
+    def __init__(self, tensor, b, h, qo_len, kv_len, causal):
+        self.tensor, self.b, self.h, self.qo_len, self.kv_len, self.causal = tensor, b, h, qo_len, kv_len, bool(causal)
+
+    @property
+    def device(self):
+        return self.tensor.device
+
+
 def stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=None):
     """A copy of a bool mask (or of the causal mask alone, ``mask=None``) that the pipelined kernel can stage: rows
     padded with False to a multiple of 16 keys, unit stride along the keys, broadcast dimensions kept as they are;
     under ``causal`` the bottom-right aligned causal mask ``n <= m + (N - M)`` is folded in (one bool mask that is
-    the conjunction of the two is what the reference's mask path would be given).  Returns the ``[b, h, M, N]``
-    view to pass as SAGE_MASK_BOOL_PADDED, or None when the copy would pass ``_STAGED_MASK_MAX_BYTES``."""
+    the conjunction of the two is what the reference's mask path would be given).  Returns a ``StagedBoolMask``,
+    or None when the copy would pass ``_STAGED_MASK_MAX_BYTES``.
+
+    ``forward`` stages on its own and keeps the last staged mask of a device (found again through the source
+    mask's storage address, version counter, shape and strides); a caller that reuses one mask over many calls
+    (all layers of a model) can stage it once here and pass the result as ``attn_mask``."""
     padded = (kv_len + 15) // 16 * 16
     if mask is None:
         bb, hh, mm = 1, 1, qo_len
     else:
+        if mask.dtype != torch.bool:
+            raise TypeError(f"stage_bool_mask takes a bool mask, got {mask.dtype}")
         m4 = mask.reshape((1,) * (4 - mask.dim()) + tuple(mask.shape))
         bb, hh, mm = m4.shape[0], m4.shape[1], (qo_len if causal else m4.shape[2])
         device = mask.device
@@ -48,7 +74,24 @@ def stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=None):
     if causal:
         rows = torch.arange(qo_len, device=buf.device).unsqueeze(1) + (kv_len - qo_len)
         live.logical_and_(torch.arange(kv_len, device=buf.device).unsqueeze(0) <= rows)
-    return live.expand(b, h, qo_len, kv_len)
+    return StagedBoolMask(live.expand(b, h, qo_len, kv_len), b, h, qo_len, kv_len, causal)
+
+
+def _staged_cached(mask, b, h, qo_len, kv_len, causal, device):
+    """``stage_bool_mask`` behind a one-entry cache per device: the same mask object contents (storage address,
+    version counter: every in-place write bumps it) under the same call shape is not staged again."""
+    if mask is None:
+        key = (None, b, h, qo_len, kv_len, causal)
+    else:
+        key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), b, h, qo_len, kv_len, causal)
+    hit = _STAGED.get(device.index)
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    staged = stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=device)
+    if staged is not None:
+        # (the source mask is kept alive with the entry: its address cannot be handed to another tensor meanwhile)
+        _STAGED[device.index] = (key, staged, mask)
+    return staged
 
 
 def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
@@ -111,14 +154,17 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
     q = q if rows_aligned(q) else q.contiguous()
     k = k if rows_aligned(k) else k.contiguous()
     v = v if rows_aligned(v) else v.contiguous()
-    q_scale = q_scale.contiguous()
-    k_scale = k_scale.contiguous()
+    if not q_scale.is_contiguous():
+        q_scale = q_scale.contiguous()
+    if not k_scale.is_contiguous():
+        k_scale = k_scale.contiguous()
 
     lib = _lib.load()
-    with torch.cuda.device(q.device):
-        o = torch.empty(q.shape, dtype=output_dtype, device=q.device)
+    dev = q.device
+    with device_guard(dev):
+        o = torch.empty(q.shape, dtype=output_dtype, device=dev)
         if return_lse:
-            lse = torch.empty([b, h_qo, qo_len], dtype=torch.float32, device=q.device)
+            lse = torch.empty([b, h_qo, qo_len], dtype=torch.float32, device=dev)
         else:
             lse = torch.empty([0], dtype=torch.float32, device="cpu")
         if b == 0 or h_qo == 0 or qo_len == 0:
@@ -129,59 +175,77 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
                 lse.fill_(float("-inf"))
             return o, lse
 
-        p = _lib.AttnParams()
-        p.q, p.k, p.v, p.out = tensor_desc(q, hnd), tensor_desc(k, hnd), tensor_desc(v, hnd), tensor_desc(o, hnd)
+        # ---- the mask as the library takes it
+        mask_kind, causal_flag, m = _lib.MASK_NONE, 1 if causal else 0, None
+        if isinstance(attn_mask, StagedBoolMask):
+            st = attn_mask
+            if (st.b, st.h, st.qo_len, st.kv_len, st.causal) != (b, h_qo, qo_len, kv_len, bool(causal)) or st.device != dev:
+                raise ValueError(
+                    f"the staged mask was made for (b, h, M, N, causal) = {(st.b, st.h, st.qo_len, st.kv_len, st.causal)} "
+                    f"on {st.device}, this call has {(b, h_qo, qo_len, kv_len, bool(causal))} on {dev}")
+            m = st.tensor
+        else:
+            if attn_mask is not None:
+                require_gpu(attn_mask, "attn_mask")
+            staged = None
+            if attn_mask is not None and attn_mask.dtype == torch.bool:
+                # bool masks run on the pipelined kernel; one that it cannot stage as it is (rows that are not 16-byte
+                # aligned, kv_len not a multiple of 16, a causal flag on top) goes there through a padded copy
+                if causal or not _bool_mask_is_direct(attn_mask.expand(b, h_qo, qo_len, kv_len), kv_len):
+                    staged = _staged_cached(attn_mask, b, h_qo, qo_len, kv_len, causal, dev)
+            elif attn_mask is None and causal and qo_len > kv_len:
+                # rows that see no key follow the reference's mask arithmetic (-1e6, whole-tile skip), which the
+                # pipelined kernel implements for mask tensors: hand it the causal mask as one
+                staged = _staged_cached(None, b, h_qo, qo_len, kv_len, True, dev)
+            if staged is not None:
+                m = staged.tensor
+            elif attn_mask is not None:
+                m = attn_mask
+                if m.dtype == torch.bool:
+                    mask_kind = _lib.MASK_BOOL
+                elif m.dtype == torch.float16:
+                    mask_kind = _lib.MASK_F16
+                elif m.dtype == torch.bfloat16:
+                    mask_kind = _lib.MASK_BF16
+                else:
+                    mask_kind = _lib.MASK_F32
+                    if m.dtype != torch.float32:  # (float64 or integer masks: the kernel adds fp32 values)
+                        m = m.float()
+                m = m.expand(b, h_qo, qo_len, kv_len)
+        if m is not None and mask_kind == _lib.MASK_NONE:  # a staged mask
+            causal_flag = 0
+            mask_kind = _lib.MASK_BOOL_PADDED_CAUSAL if causal else _lib.MASK_BOOL_PADDED
+
+        # ---- the parameter struct: built once per call shape, only pointers written afterwards
+        key = (q.shape, q.stride(), k.shape, k.stride(), v.stride(), hnd, v.dtype, output_dtype, mask_kind,
+               causal_flag, None if m is None else m.stride(), dev.index)  # (o is a fresh contiguous tensor of q's shape)
+        cache = plans()
+        plan = cache.get(key)
+        if plan is None:
+            p = _lib.AttnParams()
+            p.q, p.k, p.v, p.out = tensor_desc(q, hnd), tensor_desc(k, hnd), tensor_desc(v, hnd), tensor_desc(o, hnd)
+            p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
+            p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
+            p.v_dtype, p.out_dtype = DTYPE_CODE[v.dtype], DTYPE_CODE[output_dtype]
+            p.causal, p.mask_kind = causal_flag, mask_kind
+            if m is not None:
+                p.mask = m.data_ptr()
+                p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = m.stride()
+            p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
+            # a launch with few (batch, head, q-block) items splits its keys over more workgroups, through a workspace
+            ws_bytes = lib.sage_attn_fwd_workspace_bytes(ctypes.byref(p))
+            if ws_bytes < 0:
+                _lib.check(-1, "sage_attn_fwd_workspace_bytes")
+            plan = cache.put(key, (p, ctypes.byref(p), ws_bytes))
+        p, p_ref, ws_bytes = plan
+        p.q.ptr, p.k.ptr, p.v.ptr, p.out.ptr = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
         p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
         p.lse = lse.data_ptr() if return_lse else None
-        p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
-        p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
-        p.v_dtype, p.out_dtype = DTYPE_CODE[v.dtype], DTYPE_CODE[output_dtype]
-        p.causal = 1 if causal else 0
-        p.mask_kind = _lib.MASK_NONE
-        mask_keepalive = None
-        if attn_mask is not None:
-            require_gpu(attn_mask, "attn_mask")
-        staged = None
-        if attn_mask is not None and attn_mask.dtype == torch.bool:
-            # bool masks run on the pipelined kernel; one that it cannot stage as it is (rows that are not 16-byte
-            # aligned, kv_len not a multiple of 16, a causal flag on top) goes there through a padded copy
-            if causal or not _bool_mask_is_direct(attn_mask.expand(b, h_qo, qo_len, kv_len), kv_len):
-                staged = stage_bool_mask(attn_mask, b, h_qo, qo_len, kv_len, causal)
-        elif attn_mask is None and causal and qo_len > kv_len:
-            # rows that see no key follow the reference's mask arithmetic (-1e6, whole-tile skip), which the
-            # pipelined kernel implements for mask tensors: hand it the causal mask as one
-            staged = stage_bool_mask(None, b, h_qo, qo_len, kv_len, True, device=q.device)
-        if staged is not None:
-            p.causal = 0
-            p.mask_kind = _lib.MASK_BOOL_PADDED_CAUSAL if causal else _lib.MASK_BOOL_PADDED
-            mask_keepalive = staged
-            p.mask = staged.data_ptr()
-            p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = staged.stride()
-        elif attn_mask is not None:
-            m = attn_mask
-            if m.dtype == torch.bool:
-                p.mask_kind = _lib.MASK_BOOL
-            elif m.dtype == torch.float16:
-                p.mask_kind = _lib.MASK_F16
-            elif m.dtype == torch.bfloat16:
-                p.mask_kind = _lib.MASK_BF16
-            else:
-                p.mask_kind = _lib.MASK_F32
-                if m.dtype != torch.float32:  # (float64 or integer masks: the kernel adds fp32 values)
-                    m = m.float()
-            m = m.expand(b, h_qo, qo_len, kv_len)
-            mask_keepalive = m
-            p.mask = m.data_ptr()
-            p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = m.stride()
-        # a launch with few (batch, head, q-block) items splits its keys over more workgroups, through a workspace
-        ws_bytes = lib.sage_attn_fwd_workspace_bytes(ctypes.byref(p))
-        if ws_bytes < 0:
-            _lib.check(-1, "sage_attn_fwd_workspace_bytes")
+        p.mask = None if m is None else m.data_ptr()
+        stream = current_stream_ptr(dev)
         if ws_bytes > 0:
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
-            _lib.check(lib.sage_attn_fwd_ws(ctypes.byref(p), ws.data_ptr(), ws_bytes, current_stream_ptr(q.device)),
-                       "sage_attn_fwd_ws")
+            ws = split_workspace(dev, stream, ws_bytes)
+            _lib.check(lib.sage_attn_fwd_ws(p_ref, ws.data_ptr(), ws.numel(), stream), "sage_attn_fwd_ws")
         else:
-            _lib.check(lib.sage_attn_fwd(ctypes.byref(p), current_stream_ptr(q.device)), "sage_attn_fwd")
-        del mask_keepalive
+            _lib.check(lib.sage_attn_fwd(p_ref, stream), "sage_attn_fwd")
     return o, lse

@@ -11,7 +11,8 @@ import ctypes
 import torch
 
 from .. import _lib
-from ._common import DTYPE_CODE, current_stream_ptr, require_gpu, rows_aligned, tensor_desc
+from ._common import (DTYPE_CODE, current_stream_ptr, device_guard, plans, require_gpu, rows_aligned, split_workspace,
+                      tensor_desc)
 
 _LOG2E = 1.44269504  # literal of quant_per_block.py:87
 
@@ -43,13 +44,13 @@ def k_mean(k: torch.Tensor, tensor_layout: str = "HND") -> torch.Tensor:
     if n == 0:
         raise ValueError("k_mean of an empty sequence")
     lib = _lib.load()
-    with torch.cuda.device(k.device):
+    with device_guard(k.device):
         out = torch.empty((b, h, d), dtype=k.dtype, device=k.device)
-        ws = torch.empty(max(1, lib.sage_k_mean_workspace_bytes(b, h, n, d) // 4), dtype=torch.float32,
-                         device=k.device)
+        stream = current_stream_ptr(k.device)
+        ws = split_workspace(k.device, stream, max(4, lib.sage_k_mean_workspace_bytes(b, h, n, d)))
         desc = tensor_desc(k, hnd)
         _lib.check(lib.sage_k_mean(ctypes.byref(desc), DTYPE_CODE[k.dtype], out.data_ptr(), DTYPE_CODE[k.dtype],
-                                   b, h, n, d, ws.data_ptr(), current_stream_ptr(k.device)), "sage_k_mean")
+                                   b, h, n, d, ws.data_ptr(), stream), "sage_k_mean")
     return out.view(b, h, 1, d) if hnd else out.view(b, 1, h, d)
 
 
@@ -112,63 +113,75 @@ def _quantize(q, k, km, BLKQ, BLKK, sm_scale, tensor_layout, smooth, want_dot):
 
     lib = _lib.load()
     dot = None
-    with torch.cuda.device(q.device):
-        q_int8 = torch.empty(q.shape, dtype=torch.int8, device=q.device)
-        k_int8 = torch.empty(k.shape, dtype=torch.int8, device=k.device)
-        q_scale = torch.empty((b, h_qo, (qo_len + BLKQ - 1) // BLKQ), device=q.device, dtype=torch.float32)
-        k_scale = torch.empty((b, h_kv, (kv_len + BLKK - 1) // BLKK), device=q.device, dtype=torch.float32)
-
-        p = _lib.QuantParams()
-        p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
-        p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
-        p.blkq, p.blkk = BLKQ, BLKK
-        p.q_mul = _f32(sm_scale * _LOG2E)
-        p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
-        p.q_int8 = tensor_desc(q_int8, hnd)
-        p.k_int8 = tensor_desc(k_int8, hnd)
-        p.km = _lib.SageTensor(None, 0, 0, 0)
-        p.km_dtype = p.diff_dtype = _lib.SAGE_F32
-        stream = current_stream_ptr(q.device)
-        if fused:
-            sp = _lib.SmoothQuantParams()
-            p.in_dtype = DTYPE_CODE[q.dtype]
-            p.q = tensor_desc(q, hnd)
-            p.k = tensor_desc(k, hnd)
-            sp.quant = p
-            km_flat = torch.empty((b, h_kv, head_dim), dtype=k.dtype, device=k.device)
-            ws = torch.empty(max(1, lib.sage_k_mean_workspace_bytes(b, h_kv, kv_len, head_dim) // 4),
-                             dtype=torch.float32, device=k.device)
-            sp.km_out, sp.workspace = km_flat.data_ptr(), ws.data_ptr()
-            if want_dot:
-                dot = torch.empty((b, h_qo, qo_len), dtype=torch.float32, device=q.device)
-                sp.q_dot_km = dot.data_ptr()
-            _lib.check(lib.sage_per_block_int8_smooth_k(ctypes.byref(sp), stream), "sage_per_block_int8_smooth_k")
-            km = km_flat.view(b, h_kv, 1, head_dim) if hnd else km_flat.view(b, 1, h_kv, head_dim)
-            return q_int8, q_scale, k_int8, k_scale, km, dot
-        km_keepalive = None
-        if km is not None:
+    dev = q.device
+    with device_guard(dev):
+        q_int8 = torch.empty(q.shape, dtype=torch.int8, device=dev)
+        k_int8 = torch.empty(k.shape, dtype=torch.int8, device=dev)
+        q_scale = torch.empty((b, h_qo, (qo_len + BLKQ - 1) // BLKQ), device=dev, dtype=torch.float32)
+        k_scale = torch.empty((b, h_kv, (kv_len + BLKK - 1) // BLKK), device=dev, dtype=torch.float32)
+        kme = None
+        if km is not None and not fused:
             require_gpu(km, "km")
             if km.dtype not in DTYPE_CODE:
                 raise TypeError(f"km dtype {km.dtype} not supported (float16, bfloat16, float32)")
             kme = km.expand(k.shape)
             if not rows_aligned(kme):
                 kme = kme.contiguous()
-            km_keepalive = kme
-            p.km = tensor_desc(kme, hnd)
-            p.km_dtype = DTYPE_CODE[km.dtype]
-            p.diff_dtype = DTYPE_CODE[torch.result_type(k, km)]
-        if q.dtype == k.dtype:
+        # the parameter struct: built once per call shape, only pointers written afterwards
+        key = ("quant", q.shape, q.stride(), k.shape, k.stride(), q.dtype, k.dtype, hnd, BLKQ, BLKK, sm_scale, fused,
+               want_dot, None if kme is None else (kme.stride(), km.dtype), dev.index)
+        cache = plans()
+        plan = cache.get(key)
+        if plan is None:
+            p = _lib.QuantParams()
+            p.batch, p.heads_q, p.heads_kv = b, h_qo, h_kv
+            p.qo_len, p.kv_len, p.head_dim = qo_len, kv_len, head_dim
+            p.blkq, p.blkk = BLKQ, BLKK
+            p.q_mul = _f32(sm_scale * _LOG2E)
+            p.q_int8 = tensor_desc(q_int8, hnd)
+            p.k_int8 = tensor_desc(k_int8, hnd)
+            p.km = _lib.SageTensor(None, 0, 0, 0)
+            p.km_dtype = p.diff_dtype = _lib.SAGE_F32
             p.in_dtype = DTYPE_CODE[q.dtype]
             p.q = tensor_desc(q, hnd)
             p.k = tensor_desc(k, hnd)
-            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
+            if kme is not None:
+                p.km = tensor_desc(kme, hnd)
+                p.km_dtype = DTYPE_CODE[km.dtype]
+                p.diff_dtype = DTYPE_CODE[torch.result_type(k, km)]
+            ws_bytes = lib.sage_k_mean_workspace_bytes(b, h_kv, kv_len, head_dim) if fused else 0
+            sp = None
+            if fused:
+                sp = _lib.SmoothQuantParams()
+                sp.quant = p  # (a copy: from here on the struct inside sp is the one the call reads)
+            plan = cache.put(key, (p, sp, ctypes.byref(sp if fused else p), ws_bytes))
+        p, sp, ref, ws_bytes = plan
+        stream = current_stream_ptr(dev)
+        if fused:
+            p = sp.quant
+        p.q.ptr, p.k.ptr, p.q_int8.ptr, p.k_int8.ptr = q.data_ptr(), k.data_ptr(), q_int8.data_ptr(), k_int8.data_ptr()
+        p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
+        if fused:
+            km_flat = torch.empty((b, h_kv, head_dim), dtype=k.dtype, device=dev)
+            ws = split_workspace(dev, stream, max(ws_bytes, 4))
+            sp.km_out, sp.workspace = km_flat.data_ptr(), ws.data_ptr()
+            if want_dot:
+                dot = torch.empty((b, h_qo, qo_len), dtype=torch.float32, device=dev)
+                sp.q_dot_km = dot.data_ptr()
+            _lib.check(lib.sage_per_block_int8_smooth_k(ref, stream), "sage_per_block_int8_smooth_k")
+            km = km_flat.view(b, h_kv, 1, head_dim) if hnd else km_flat.view(b, 1, h_kv, head_dim)
+            return q_int8, q_scale, k_int8, k_scale, km, dot
+        if kme is not None:
+            p.km.ptr = kme.data_ptr()
+        if q.dtype == k.dtype:
+            _lib.check(lib.sage_per_block_int8(ref, stream), "sage_per_block_int8")
         else:
-            null = _lib.SageTensor(None, 0, 0, 0)
-            p.in_dtype, p.q, p.k = DTYPE_CODE[q.dtype], tensor_desc(q, hnd), null
-            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
-            p.in_dtype, p.q, p.k = DTYPE_CODE[k.dtype], null, tensor_desc(k, hnd)
-            _lib.check(lib.sage_per_block_int8(ctypes.byref(p), stream), "sage_per_block_int8")
-        del km_keepalive
+            kp = p.k.ptr
+            p.in_dtype, p.k.ptr = DTYPE_CODE[q.dtype], None
+            _lib.check(lib.sage_per_block_int8(ref, stream), "sage_per_block_int8")
+            p.in_dtype, p.q.ptr, p.k.ptr = DTYPE_CODE[k.dtype], None, kp
+            _lib.check(lib.sage_per_block_int8(ref, stream), "sage_per_block_int8")
+        del kme
     if want_dot and km is not None:  # (mixed dtypes or an unusual head_dim: the dot product is taken by torch)
         qh, kmh = (q, km) if hnd else (q.transpose(1, 2), km.transpose(1, 2))
         groups = h_qo // h_kv

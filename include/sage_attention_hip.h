@@ -75,7 +75,7 @@ int sage_per_block_int8(const sage_quant_params* p, void* stream);
  *   out          out_dtype (SAGE_F16 / SAGE_BF16 / SAGE_F32), own strides
  *   lse          optional [B, Hq, M] fp32 contiguous, base-2 log-sum-exp (:124-127); NULL = none
  *   mask         optional [B, Hq, M, N] through 4 strides (elements, 0 = broadcast);
- *                SAGE_MASK_BOOL: 1 byte per element, 1 = keep, 0 = hide (:33-36,48); other byte values are not allowed;
+ *                SAGE_MASK_BOOL: 1 byte per element, non-zero = keep, 0 = hide (:33-36,48), on every route;
  *                SAGE_MASK_BOOL_PADDED: the same, and the caller guarantees that every mask row can be read up to the
  *                next multiple of 16 bytes past kv_len and holds zeros there (a staging copy with padded rows): with
  *                16-byte aligned rows such a mask runs on the pipelined kernel for any kv_len, where a plain

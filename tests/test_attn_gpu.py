@@ -369,6 +369,90 @@ def test_bool_mask_kinds_through_the_c_abi(n, gpu_device):
     assert lib.sage_attn_fwd(ctypes.byref(p), None) == -1 and b"mask_kind" in lib.sage_hip_last_error()
 
 
+@pytest.mark.parametrize("n", [96, 70])
+def test_bool_mask_bytes_other_than_one(n, gpu_device):
+    """A mask whose visible entries are stored as 0xFF (or any other non-zero byte: a uint8 tensor viewed as bool, a
+    C caller) gives the results of the same mask stored as 0 / 1 on every route: the pipelined kernel as the
+    mask is (n = 96), through the host's padded copy (n = 70), and the general kernel (C ABI, odd row starts)."""
+    import ctypes
+
+    from flagattention_amd import _lib
+    from flagattention_amd.sage_attention._common import DTYPE_CODE, tensor_desc
+
+    b, h, m, d = 1, 2, 200, 128
+    q8, qs, k8, ks, v = (t.to(gpu_device) for t in _quantized(48, b, h, h, m, n, d, torch.bfloat16))
+    mask = _mask_case("holes", b, h, m, n, 17).to(gpu_device)
+    g = torch.Generator().manual_seed(3)
+    odd_bytes = torch.randint(2, 256, mask.shape, generator=g, dtype=torch.int32).to(torch.uint8).to(gpu_device)
+    loud = torch.where(mask, odd_bytes, torch.zeros_like(odd_bytes)).view(torch.bool)  # same truth values, bytes 2 .. 255
+    assert int(loud.view(torch.uint8).max()) > 1
+    want, want_lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=mask, return_lse=True, output_dtype=torch.float32)
+    got, got_lse = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=loud, return_lse=True, output_dtype=torch.float32)
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    # the general kernel: SAGE_MASK_BOOL on rows that start at odd addresses
+    lib = _lib.load()
+    store = torch.zeros(b, h, m, n + 3, dtype=torch.uint8, device=gpu_device)
+    view = store[..., 1:1 + n]
+    view.copy_(loud.view(torch.uint8))
+    o = torch.empty(q8.shape, dtype=torch.float32, device=gpu_device)
+    lse = torch.empty(b, h, m, dtype=torch.float32, device=gpu_device)
+    p = _lib.AttnParams()
+    p.q, p.k, p.v, p.out = (tensor_desc(t, True) for t in (q8, k8, v, o))
+    p.q_scale, p.k_scale, p.lse = qs.data_ptr(), ks.data_ptr(), lse.data_ptr()
+    p.batch, p.heads_q, p.heads_kv, p.qo_len, p.kv_len, p.head_dim = b, h, h, m, n, d
+    p.v_dtype, p.out_dtype = DTYPE_CODE[torch.bfloat16], DTYPE_CODE[torch.float32]
+    p.mask_kind, p.mask = _lib.MASK_BOOL, view.data_ptr()
+    p.mask_stride_b, p.mask_stride_h, p.mask_stride_m, p.mask_stride_n = view.stride()
+    assert lib.sage_attn_fwd(ctypes.byref(p), torch.cuda.current_stream().cuda_stream) == 0, lib.sage_hip_last_error()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(o, want, atol=5e-3, rtol=1e-2)
+    torch.testing.assert_close(lse, want_lse, atol=6e-3, rtol=1e-4)
+
+
+def test_a_bool_mask_is_staged_once(gpu_device):
+    """A mask the pipelined kernel cannot read as it is (kv_len not a multiple of 16) is copied into its padded
+    form on the first call only: the second call with the same mask allocates nothing beyond its outputs and gives
+    the same bits; a mask staged by hand (stage_bool_mask) is taken as it is; an in-place change of the mask is
+    seen; a staged mask made for another call shape is refused."""
+    from flag_attn import sage_attention as sa
+
+    b, hq, hkv, m, n = 2, 4, 2, 300, 500
+    q8, qs, k8, ks, v = (t.to(gpu_device) for t in _quantized(49, b, hq, hkv, m, n, 128, torch.bfloat16))
+    mask = _mask_case("random", 1, 1, m, n, 19).to(gpu_device)
+    kw = dict(return_lse=True, output_dtype=torch.float32)
+    o1, lse1 = sa.forward(q8, k8, v, qs, ks, attn_mask=mask, **kw)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(gpu_device)
+    o2, lse2 = sa.forward(q8, k8, v, qs, ks, attn_mask=mask, **kw)
+    torch.cuda.synchronize()
+    grown = torch.cuda.memory_allocated(gpu_device) - before
+    outputs = o2.numel() * 4 + lse2.numel() * 4
+    assert grown <= outputs + 1024, (grown, outputs)  # (the allocator rounds sizes up to 512 bytes)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    expected, expected_lse = C.attention_blockwise(q8.cpu(), k8.cpu(), v.cpu(), qs.cpu(), ks.cpu(),
+                                                   attn_mask=mask.cpu().expand(b, hq, m, n))
+    _check_masked(o2, lse2, expected, expected_lse, "cached staging")
+    staged = sa.stage_bool_mask(mask, b, hq, m, n, False)
+    assert isinstance(staged, sa.StagedBoolMask) and staged.tensor.stride(1) == 0  # broadcast over heads kept
+    o3, lse3 = sa.forward(q8, k8, v, qs, ks, attn_mask=staged, **kw)
+    assert torch.equal(o1, o3) and torch.equal(lse1, lse3)
+    with pytest.raises(ValueError, match="staged mask was made for"):
+        sa.forward(q8, k8, v, qs, ks, attn_mask=staged, causal=True, **kw)
+    mask[..., : n // 2] = False  # in place: the version counter of the tensor moves, the copy is made again
+    o4, lse4 = sa.forward(q8, k8, v, qs, ks, attn_mask=mask, **kw)
+    expected, expected_lse = C.attention_blockwise(q8.cpu(), k8.cpu(), v.cpu(), qs.cpu(), ks.cpu(),
+                                                   attn_mask=mask.cpu().expand(b, hq, m, n))
+    _check_masked(o4, lse4, expected, expected_lse, "after an in-place change")
+    # causal with more queries than keys and no mask: the causal mask is staged once per (M, N) as well
+    qc, qsc, kc, ksc, vc = (t.to(gpu_device) for t in _quantized(50, 1, 2, 2, 400, 150, 64, torch.float16))
+    sa.forward(qc, kc, vc, qsc, ksc, causal=True)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(gpu_device)
+    oc, _ = sa.forward(qc, kc, vc, qsc, ksc, causal=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated(gpu_device) - before <= oc.numel() * 2 + 1024
+
+
 @pytest.mark.parametrize("pattern", sorted(_SCALE_PATTERNS))
 def test_bool_mask_with_row_maximum_that_moves(pattern, gpu_device):
     m, n = 320, 768

@@ -151,7 +151,9 @@ def test_bool_mask_staging_copy():
                                         ((2, 3, 9, 70), True, (2, 3, 9, 70)), ((9, 70), True, (2, 3, 9, 70)),
                                         ((1, 1, 12, 7), True, (1, 2, 12, 7)), ((3, 1, 64), False, (2, 3, 1, 64))]:
         mask = torch.rand(shape, generator=g) > 0.4
-        staged = stage_bool_mask(mask, b, h, m, n, causal)
+        st = stage_bool_mask(mask, b, h, m, n, causal)
+        assert (st.b, st.h, st.qo_len, st.kv_len, st.causal) == (b, h, m, n, causal)
+        staged = st.tensor
         want = mask.expand(b, h, m, n)
         if causal:
             want = want & (torch.arange(n)[None, :] <= torch.arange(m)[:, None] + (n - m))
@@ -163,11 +165,37 @@ def test_bool_mask_staging_copy():
         for dim, size in enumerate(mask.reshape((1,) * (4 - mask.dim()) + tuple(mask.shape)).shape[:2]):
             if size == 1 and (b, h)[dim] > 1:
                 assert staged.stride(dim) == 0  # broadcast over batch / heads stays a broadcast
-    only_causal = stage_bool_mask(None, 1, 2, 12, 7, True, device="cpu")
+    only_causal = stage_bool_mask(None, 1, 2, 12, 7, True, device="cpu").tensor
     assert torch.equal(only_causal[0, 1], torch.arange(7)[None, :] <= torch.arange(12)[:, None] - 5)
     aligned = torch.ones(2, 3, 8, 64, dtype=torch.bool)
     assert _bool_mask_is_direct(aligned, 64) and not _bool_mask_is_direct(aligned[..., :60], 60)
     assert not _bool_mask_is_direct(aligned.transpose(2, 3), 8)
+
+
+def test_staged_mask_cache_key_and_cap(monkeypatch):
+    """The one-entry cache behind forward's staging: the same mask under the same call shape is staged once; an
+    in-place write (version counter), another shape or another causal flag stages again; the source mask is kept
+    alive with the entry, so its address cannot come back as another tensor.  Copies above the cap are refused."""
+    import torch
+
+    from flagattention_amd.sage_attention import attention as A
+
+    dev = torch.device("cpu")
+    A._STAGED.clear()
+    mask = torch.rand((1, 1, 9, 37)) > 0.5
+    s1 = A._staged_cached(mask, 2, 3, 9, 37, False, dev)
+    assert A._staged_cached(mask, 2, 3, 9, 37, False, dev) is s1
+    assert A._staged_cached(mask.view(1, 1, 9, 37), 2, 3, 9, 37, False, dev) is s1  # another view of the same data
+    assert A._STAGED[None][2] is mask
+    mask[0, 0, 0, 0] = not bool(mask[0, 0, 0, 0])  # in-place write: staged again, with the new value
+    s2 = A._staged_cached(mask, 2, 3, 9, 37, False, dev)
+    assert s2 is not s1 and torch.equal(s2.tensor, mask.expand(2, 3, 9, 37))
+    assert A._staged_cached(mask, 2, 3, 9, 37, True, dev) is not s2
+    assert A._staged_cached(None, 1, 2, 12, 7, True, dev) is A._staged_cached(None, 1, 2, 12, 7, True, dev)
+    monkeypatch.setattr(A, "_STAGED_MASK_MAX_BYTES", 1024)
+    assert A.stage_bool_mask(torch.ones((2, 3, 9, 37), dtype=torch.bool), 2, 3, 9, 37, False) is None
+    assert A.stage_bool_mask(torch.ones((1, 1, 9, 37), dtype=torch.bool), 2, 3, 9, 37, False) is not None
+    A._STAGED.clear()
 
 
 def test_python_api_errors_on_cpu():

@@ -52,6 +52,24 @@ def test_no_alloc_k_mean_matches_workspace_variant(gpu_device):
         assert torch.equal(got.cpu().view(torch.uint8), oracle.view(torch.uint8))
 
 
+@pytest.mark.parametrize("n", [32768, 32768 - 5])
+def test_no_alloc_k_mean_at_the_last_byte_of_its_scratch(n, gpu_device):
+    """A launch that fills the built-in array to its last byte (1 x 32 heads x 512 chunks x 128 channels fp32 =
+    8 MiB), with a whole and with a ragged last chunk: bit for bit the workspace variant, and the oracle on the
+    first and the last head (whose partials lie at the two ends of the array)."""
+    from flagattention_amd import _lib
+
+    lib = _lib.load()
+    assert lib.sage_k_mean_workspace_bytes(1, 32, n, 128) == _lib.K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES
+    g = torch.Generator(device=gpu_device).manual_seed(7)
+    k = (torch.randn(1, 32, n, 128, generator=g, device=gpu_device) + 0.5).to(torch.bfloat16)
+    want, got = _both(k, "HND", gpu_device)
+    assert torch.equal(want.view(torch.uint8), got.view(torch.uint8))
+    for head in (0, 31):
+        oracle = C.k_mean_fixed_order(k[:, head:head + 1].cpu(), "HND").reshape(128)
+        assert torch.equal(got[0, head].cpu().view(torch.uint8), oracle.view(torch.uint8)), head
+
+
 def test_no_alloc_k_mean_rejects_what_does_not_fit(gpu_device):
     from flagattention_amd import _lib
 
