@@ -40,7 +40,8 @@ struct AttnArgs {
     int32_t total_wg;
     int32_t mask_vec;  // mask rows are contiguous along the keys and every group of four entries is naturally aligned
     int32_t mask_dt;   // storage type of an additive mask (SAGE_F32 / SAGE_F16 / SAGE_BF16)
-    int32_t mask_padded;  // bool mask rows are readable, and zero, up to the next multiple of 16 bytes past kv_len
+    int32_t mask_additive;  // the mask tensor is additive (entries of type mask_dt), not bool
+    int32_t mask_padded;  // mask rows are readable (bool: and zero) up to the next multiple of 16 bytes past kv_len
     int32_t mask_causal;  // the bool mask is False wherever n > m + (kv_len - qo_len): tiles beyond need no visit
     // Heads that take turns within one q-block in the order of the workgroups (1: a head's q-blocks follow each
     // other).  Under a mask shared by the heads, head_tile heads x several q-blocks run side by side on an XCD, so
@@ -102,9 +103,11 @@ int64_t key_split_workspace_bytes(int nsplit, int64_t batch, int64_t heads_q, in
 void apply_key_split(AttnArgs& a, int nsplit, int64_t batch, int head_dim, void* workspace);
 int launch_split_combine(const AttnArgs& split, const AttnArgs& whole, int head_dim, int64_t batch, hipStream_t stream);
 
-// The same kernel under a bool mask tensor, where fast_serves_mask() says so (a.mask set, MODE_MASK_BOOL).
-bool fast_serves_mask(const AttnArgs& a);
+// The same kernel under a bool mask tensor or an additive fp16 / bf16 one, where fast_serves_mask() says so (a.mask
+// set; esz: bytes per mask entry).
+bool fast_serves_mask(const AttnArgs& a, int esz);
 int launch_fast_masked(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream);
+int launch_fast_additive(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream);
 
 // The same kernel on 16-bit Q and K (dense attention); causal with any qo_len / kv_len.
 int launch_flash(const AttnArgs& a, int head_dim, int dtype, bool causal, hipStream_t stream);

@@ -115,16 +115,41 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 // step into that path until the row has seen a key.  a.mask_causal: the caller folded the causal mask into the
 // tensor, so tiles beyond the causal limit of the workgroup's last row need no visit.  Additive masks and masks
 // with unaligned rows stay with the general kernel (attn_fwd.hip).
-constexpr int kMaskSlots = 3;                       // steps of mask bytes resident per wave
-constexpr int kMaskWaveBytes = 32 * BN;            // 32 rows x 64 keys x 1 byte
-constexpr int kMaskBytes = kMaskSlots * kFastWaves * kMaskWaveBytes;
+//
+// MT (the type of a mask entry): void = no mask tensor, bool = the bool mask above, _Float16 / __bf16 = an additive
+// mask tensor in that storage type (attn_qk_int8_per_block.py:37-38,49-50: score + mask entry, no tile is skipped).
+// Staged like the bool mask, 32 x 64 entries of 2 bytes per wave and step, two steps resident (with the four K/V
+// tiles that fills the 160 KB of the CU at head_dim 128: the entries of step j + 1 are requested during the
+// vector phase of step j, ahead of that phase's K/V loads, and waited for at the end of the matrix phase that
+// follows).  The entry is added to the exponent of its score: fma(score, scale, entry - m).  Rows start from the
+// reference point -inf like those of the bool instance, so the first step of every row runs the path that redoes a
+// step, which takes the row maximum of score * scale + entry; so does a ragged last tile, whose keys past kv_len
+// score -1e6 there as in the reference (mask entries read as -1e6, K as zeros).
+template <typename MT> struct MaskT { static constexpr int BYTES = sizeof(MT), SLOTS = 2; static constexpr bool ON = true, ADD = true; };
+template <> struct MaskT<void> { static constexpr int BYTES = 1, SLOTS = 1; static constexpr bool ON = false, ADD = false; };
+template <> struct MaskT<bool> { static constexpr int BYTES = 1, SLOTS = 3; static constexpr bool ON = true, ADD = false; };
 constexpr float kMaskedScore = -1.0e6f;            // what the reference adds to the score of a hidden key
 
-template <int D, typename VT, bool CAUSAL, int QB, bool MASK = false>
+// an additive mask entry (16 bits, the low or the high half of a word) as fp32
+template <typename MT> __device__ __forceinline__ float mask_entry(unsigned word, int hi);
+template <> __device__ __forceinline__ float mask_entry<__bf16>(unsigned word, int hi) {
+    return __builtin_bit_cast(float, hi ? (word & 0xffff0000u) : (word << 16));
+}
+template <> __device__ __forceinline__ float mask_entry<_Float16>(unsigned word, int hi) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)(hi ? (word >> 16) : (word & 0xffffu)));
+}
+
+template <int D, typename VT, bool CAUSAL, int QB, typename MT = void>
 __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast_kernel(AttnArgs a, int nq2) {
     using F = FT<D, QB>;
     constexpr bool INT8 = QB == 1;
-    static_assert(!MASK || (CAUSAL && INT8), "the mask instance builds on the key-hiding int8 instance");
+    constexpr bool MASK = MaskT<MT>::ON;         // a mask tensor is staged
+    constexpr bool MADD = MaskT<MT>::ADD;        // ... an additive one (else bool)
+    constexpr int kMaskSlots = MaskT<MT>::SLOTS;                 // steps of mask entries resident per wave
+    constexpr int kMaskWaveBytes = 32 * BN * MaskT<MT>::BYTES;   // 32 rows x 64 keys
+    constexpr int kMaskInstr = kMaskWaveBytes / 1024;            // loads per wave and step
+    constexpr int kMaskBytes = kMaskSlots * kFastWaves * kMaskWaveBytes;
+    static_assert(!MASK || (CAUSAL && INT8), "the mask instances build on the key-hiding int8 instance");
     constexpr float BIAS = INT8 ? kBias : 0.0f;  // what the bits of a fresh score accumulator read as a float
     using PVT = PV<VT>;
     using vec16 = typename PVT::vec;
@@ -276,7 +301,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                   lds0 + F::V_BASE + vbuf * F::V_BYTES + 1024 * (wave_u + kFastWaves * ev));
         }
     };
-    constexpr int NDMA = F::NK + F::NV + (MASK ? 2 : 0);  // loads per wave per step
+    constexpr int NDMA = F::NK + F::NV + (MASK ? kMaskInstr : 0);  // loads per wave per step
     constexpr int NDMA_KV = F::NK + F::NV;
 
     // ---- mask staging (MASK): the wave's 32 rows x 64 keys of step t go to slot t % 3 of its own 2 KB slices, row
@@ -285,28 +310,43 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     //      of the row number: rows 4 apart, whose pieces would share banks, read different pieces.  Rows past
     //      qo_len re-read the last row, chunks past kv_len (last tile of a kv_len that is not a multiple of 64)
     //      the last chunk: duplicates of valid entries, so neither the products nor the look for a visible key see anything new.
+    //      Additive 16-bit entries: 128 bytes per row, eight lanes per row, instruction e carries rows 8 e .. 8 e + 7;
+    //      the eight chunks of a row are XOR-swizzled in pairs with bits 0-1 of the row number (a lane reads the two
+    //      chunks of a 16-key slice with one instruction: they stay neighbours).
     const unsigned char* mask_row0 = nullptr;  // uniform: this wave's first mask row
-    unsigned m_goff[2] = {0, 0}, m_goff_last[2] = {0, 0};
+    constexpr int MB = MaskT<MT>::BYTES;       // bytes per mask entry
+    constexpr int kMaskLPR = BN * MB / 16;     // lanes (16-byte chunks) per staged row: 4 | 8
+    unsigned m_goff[kMaskInstr] = {}, m_goff_last[kMaskInstr] = {};
     if constexpr (MASK) {
         const int row_first = min(m0 + 32 * wave_u, a.M - 1);
-        mask_row0 = static_cast<const unsigned char*>(a.mask) + (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)row_first * a.ms_m;
-        const int last_chunk = ((kv_len - 1) % BN) / 16;
+        mask_row0 = static_cast<const unsigned char*>(a.mask) + ((int64_t)b * a.ms_b + (int64_t)h * a.ms_h + (int64_t)row_first * a.ms_m) * MB;
+        const int last_chunk = ((kv_len - 1) % BN) * MB / 16;
 #pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const int r = min(16 * e + (lane >> 2), a.M - 1 - row_first);
-            const int chunk = (lane & 3) ^ ((lane >> 4) & 3);  // (bits 2-3 of the row number 16 e + lane / 4)
-            m_goff[e] = (unsigned)(r * (int)a.ms_m + 16 * chunk);
-            m_goff_last[e] = (unsigned)(r * (int)a.ms_m + 16 * min(chunk, last_chunk));
+        for (int e = 0; e < kMaskInstr; e++) {
+            const int rl = (64 / kMaskLPR) * e + lane / kMaskLPR;  // row of the wave's tile
+            const int r = min(rl, a.M - 1 - row_first);
+            const int chunk = MADD ? (lane % kMaskLPR) ^ (2 * (rl & 3))
+                                   : (lane & 3) ^ ((lane >> 4) & 3);  // (bits 2-3 of the row number 16 e + lane / 4)
+            m_goff[e] = (unsigned)((r * (int)a.ms_m) * MB + 16 * chunk);
+            m_goff_last[e] = (unsigned)((r * (int)a.ms_m) * MB + 16 * min(chunk, last_chunk));
         }
     }
     auto dma_mask = [&](int tile, int slot) {
         if constexpr (MASK) {
             const bool cut = ragged && tile == nk - 1;
 #pragma unroll
-            for (int e = 0; e < 2; e++)
-                dma16(mask_row0 + (int64_t)tile * BN, cut ? m_goff_last[e] : m_goff[e],
+            for (int e = 0; e < kMaskInstr; e++)
+                dma16(mask_row0 + (int64_t)tile * BN * MB, cut ? m_goff_last[e] : m_goff[e],
                       lds0 + F::TOTAL + (slot * kFastWaves + wave_u) * kMaskWaveBytes + 1024 * e);
         }
+    };
+    // (additive) the lane's entries of 16-key slice tp of a staged step: four words, the entries of score registers
+    // 8 (tp & 1) + 0 .. 3 (two words) and + 4 .. 7 (two words) of tile tp >> 1
+    auto mask_entries = [&](int slot, int tp, unsigned (&w)[4]) {
+        const unsigned char* row = smem + F::TOTAL + (slot * kFastWaves + wave) * kMaskWaveBytes + l32 * (BN * MB) + 8 * half;
+        const v2u* piece = reinterpret_cast<const v2u*>(row + 32 * (tp ^ (l32 & 3)));
+        const v2u lo = piece[0], hi = piece[2];
+        w[0] = lo[0]; w[1] = lo[1]; w[2] = hi[0]; w[3] = hi[1];
     };
     // The lane's mask bytes of 16-key slice tp of a staged step: two words, keys 8 g + 4 half .. + 3 for the even and
     // the odd g of the slice (the keys of score registers 8 (tp & 1) .. + 3 and + 4 .. + 7 of tile tp >> 1).
@@ -456,7 +496,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     // from here on k_fetch / v_fetch point at the tiles fetched during step 0: K of step 3, V of step 2
     if (nsteps > 3) { k_fetch += k_tile_bytes; k_tile++; }
     dma_mask(0, 0);
-    dma_mask(max(min(1, nsteps - 1), 0), 1);  // (nsteps = 0: a workgroup that sees no key; tile 0 exists all the same)
+    if constexpr (kMaskSlots == 3) dma_mask(max(min(1, nsteps - 1), 0), 1);  // (nsteps = 0: a workgroup that sees no key; tile 0 exists all the same)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct-to-LDS loads have landed
     __syncthreads();
     sbuf[0][0] = qk_tile(smem, 0);
@@ -532,21 +572,33 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
 
         // The direct-to-LDS loads are issued from the VALU phase, where a stalled issue delays no matrix
         // instruction.
-        sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
         const int mslot_next = mslot == kMaskSlots - 1 ? 0 : mslot + 1;
-        dma_mask(min(step + 2, nsteps - 1), mslot_next == kMaskSlots - 1 ? 0 : mslot_next + 1);  // the mask bytes of step + 2
+        // (additive: the entries of step + 1, into the slot that step - 1 left; ahead of the K/V loads, because they
+        // are the ones waited for first: at the end of the coming matrix phase)
+        if constexpr (MADD) dma_mask(min(step + 1, nsteps - 1), mslot_next);
+        sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
+        if constexpr (MASK && !MADD) dma_mask(min(step + 2, nsteps - 1), mslot_next == kMaskSlots - 1 ? 0 : mslot_next + 1);  // the mask bytes of step + 2
         vec16 pf[4];
         float lsum = 0.0f;
         const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
-        unsigned mw[2][2] = {{0, 0}, {0, 0}};  // (MASK) the lane's mask bytes of the 16-key slice in work and of the next one
-        if constexpr (MASK) mask_words(mslot, 0, mw[0][0], mw[0][1]);
+        unsigned mw[2][2] = {{0, 0}, {0, 0}};  // (bool mask) the lane's mask bytes of the 16-key slice in work and of the next one
+        unsigned me[2][4] = {};                // (additive mask) the lane's entries of the slice in work and of the next one
+        if constexpr (MASK && !MADD) mask_words(mslot, 0, mw[0][0], mw[0][1]);
+        if constexpr (MADD) mask_entries(mslot, 0, me[0]);
         auto exp_unit = [&](auto uc) {  // two scores -> two 16-bit P values
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
             const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
-            float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, neg_m));
-            float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, neg_m));
-            if constexpr (MASK) {
+            float t0 = neg_m, t1 = neg_m;
+            if constexpr (MADD) {  // the mask entry joins the exponent: score * scale + entry - m
+                if constexpr (w == 0 && tp < 3) mask_entries(mslot, tp + 1, me[(tp + 1) & 1]);
+                const unsigned word = me[tp & 1][w];
+                t0 += mask_entry<MT>(word, 0);
+                t1 += mask_entry<MT>(word, 1);
+            }
+            float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b0), sc_e, t0));
+            float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(b1), sc_e, t1));
+            if constexpr (MASK && !MADD) {
                 // P of a hidden key is 0.  An overflowed P times 0 is NaN: the row sum then
                 // sends the step into the path that redoes it.
                 if constexpr (w == 0 && tp < 3) mask_words(mslot, tp + 1, mw[(tp + 1) & 1][0], mw[(tp + 1) & 1][1]);
@@ -590,6 +642,52 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         v4f sum4 = {0.0f, 0.0f, 0.0f, 0.0f};
         unsigned long long large = 0;
         auto redo_if_large = [&]() {
+            if constexpr (MADD) {
+                // a ragged last tile always comes here: its keys past kv_len score -1e6 (the reference reads their
+                // mask entries as -1e6 and their K as zeros), which only this path accounts for
+                if (large != 0 || (ragged && step == nk - 1)) {
+                    float raw = -INFINITY;
+                    float past_end = 0.0f;  // number of the lane's keys of this step that lie past kv_len
+                    sfor<4>([&](auto tc) {
+                        constexpr int tp = decltype(tc)::value, kt = tp >> 1;
+                        unsigned w4[4];
+                        mask_entries(mslot, tp, w4);
+#pragma unroll
+                        for (int c = 0; c < 8; c++) {
+                            const int i = 8 * (tp & 1) + c;
+                            const int bits = sbuf[P][kt][i];
+                            const float x = as_f(bits);
+                            float sv = __builtin_fmaf(folded ? x - BIAS : x, sc_e, mask_entry<MT>(w4[c >> 1], c & 1));
+                            if (x == -INFINITY) {  // past kv_len
+                                sv = -INFINITY;
+                                past_end += 1.0f;
+                            }
+                            sbuf[P][kt][i] = __builtin_bit_cast(int, sv);
+                            raw = fmaxf(raw, sv);
+                        }
+                    });
+                    if (past_end > 0.0f) raw = fmaxf(raw, kMaskedScore);
+                    const float m_new = fmaxf(m_i, row_pair_max(raw));
+                    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);  // 0 for a row that had no reference point yet
+                    l_i *= alpha;
+                    m_i = m_new;
+#pragma unroll
+                    for (int dt = 0; dt < F::DTILES; dt++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+                    lsum = 0.0f;
+                    sfor<16>([&](auto uc) {
+                        constexpr int u = decltype(uc)::value;
+                        constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
+                        const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
+                        pf[tp][2 * w] = (VT)__builtin_amdgcn_exp2f(as_f(b0) - m_i);
+                        pf[tp][2 * w + 1] = (VT)__builtin_amdgcn_exp2f(as_f(b1) - m_i);
+                        lsum = PVT::dot2_ones(pf[tp], w, lsum);
+                    });
+                    lsum = __builtin_fmaf(past_end, __builtin_amdgcn_exp2f(kMaskedScore - m_i), lsum);
+                }
+                return;
+            }
             if constexpr (MASK) {
                 if (large != 0 && !tile_has_visible_key(mslot)) {
                     // no visible key for this 128-row block in this tile: the reference skips it.  (Rows without a
@@ -762,6 +860,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         if (step + 4 < nsteps) { k_fetch += k_tile_bytes; k_tile++; }  // next iteration fetches K of step+4, V of step+3
         if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
         __builtin_amdgcn_s_setprio(0);
+        // (additive mask: the entries of the next step, requested ahead of this step's K/V loads, have landed)
+        if constexpr (MADD) __builtin_amdgcn_s_waitcnt(0x0F70 | NDMA_KV);
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
         __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
         __builtin_amdgcn_sched_barrier(0);

@@ -27,7 +27,7 @@ int launch_masked(const AttnArgs& a, hipStream_t stream) {
     const int nq2 = (a.M + kFastRows - 1) / kFastRows;
     b.total_wg = (int)((int64_t)a.total_wg / a.nq * nq2);
     dim3 grid((unsigned)b.total_wg), block(kFastThreads);
-    hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1, true>), grid, block, 0, stream, b, nq2);
+    hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1, bool>), grid, block, 0, stream, b, nq2);
     return check_launch("sage_attn_fwd_fast_kernel (bool mask)");
 }
 
@@ -36,13 +36,16 @@ int launch_masked(const AttnArgs& a, hipStream_t stream) {
 // A bool mask tensor the pipelined kernel can stage with 16-byte loads: contiguous along the keys, every row start
 // 16-byte aligned, no load that reaches past the end of a row (kv_len a multiple of 16, or rows that the caller
 // padded with zeros to one), no causal flag on top.
-bool fast_serves_mask(const AttnArgs& a) {
-    return a.mask != nullptr && !a.causal && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 && a.ms_b % 16 == 0 &&
-           a.ms_h % 16 == 0 && a.ms_m % 16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 26) &&
-           (a.N % 16 == 0 || a.mask_padded);
+// (esz: bytes per mask entry, 1 for bool masks, 2 for additive fp16 / bf16 ones; fp32 masks are not staged)
+bool fast_serves_mask(const AttnArgs& a, int esz) {
+    const int per16 = 16 / esz;  // entries per 16-byte load
+    return a.mask != nullptr && !a.causal && (esz == 1 || esz == 2) && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 &&
+           a.ms_b % per16 == 0 && a.ms_h % per16 == 0 && a.ms_m % per16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 25) &&
+           (a.N % per16 == 0 || a.mask_padded);
 }
 
 int launch_fast_masked(const AttnArgs& a, int head_dim, int v_dtype, hipStream_t stream) {
+    if (a.mask_additive) return launch_fast_additive(a, head_dim, v_dtype, stream);
     if (head_dim == 128)
         return v_dtype == SAGE_BF16 ? launch_masked<128, __bf16>(a, stream) : launch_masked<128, _Float16>(a, stream);
     return v_dtype == SAGE_BF16 ? launch_masked<64, __bf16>(a, stream) : launch_masked<64, _Float16>(a, stream);
