@@ -10,7 +10,7 @@ ABI_VERSION = 3
 
 SAGE_F16, SAGE_BF16, SAGE_F32 = 0, 1, 2
 MASK_NONE, MASK_BOOL, MASK_F32, MASK_F16, MASK_BF16, MASK_BOOL_PADDED, MASK_BOOL_PADDED_CAUSAL = 0, 1, 2, 3, 4, 5, 6
-MASK_F16_PADDED, MASK_BF16_PADDED = 7, 8
+MASK_F16_PADDED, MASK_BF16_PADDED, MASK_F32_PADDED = 7, 8, 9
 K_MEAN_NOALLOC_MAX_WORKSPACE_BYTES = 8 * 1024 * 1024
 
 c_i64 = ctypes.c_int64

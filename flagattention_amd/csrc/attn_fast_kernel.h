@@ -125,7 +125,10 @@ __device__ __forceinline__ typename PV<VT>::vec tr_pair(const unsigned char* p0,
 // reference point -inf like those of the bool instance, so the first step of every row runs the path that redoes a
 // step, which takes the row maximum of score * scale + entry; so does a ragged last tile, whose keys past kv_len
 // score -1e6 there as in the reference (mask entries read as -1e6, K as zeros).
-template <typename MT> struct MaskT { static constexpr int BYTES = sizeof(MT), SLOTS = 2; static constexpr bool ON = true, ADD = true; };
+// fp32 entries: 8 KB per wave and step, ONE step resident (two would not fit beside the K/V tiles): the entries of
+// step j + 1 are requested at the end of the vector phase of step j, once its last entry has been read, and waited for
+// at the end of the matrix phase that follows; the path that redoes a step reads its entries from memory again.
+template <typename MT> struct MaskT { static constexpr int BYTES = sizeof(MT), SLOTS = sizeof(MT) == 4 ? 1 : 2; static constexpr bool ON = true, ADD = true; };
 template <> struct MaskT<void> { static constexpr int BYTES = 1, SLOTS = 1; static constexpr bool ON = false, ADD = false; };
 template <> struct MaskT<bool> { static constexpr int BYTES = 1, SLOTS = 3; static constexpr bool ON = true, ADD = false; };
 constexpr float kMaskedScore = -1.0e6f;            // what the reference adds to the score of a hidden key
@@ -145,6 +148,7 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr bool INT8 = QB == 1;
     constexpr bool MASK = MaskT<MT>::ON;         // a mask tensor is staged
     constexpr bool MADD = MaskT<MT>::ADD;        // ... an additive one (else bool)
+    constexpr bool MF32 = MADD && MaskT<MT>::BYTES == 4;   // ... with fp32 entries (else 16-bit ones)
     constexpr int kMaskSlots = MaskT<MT>::SLOTS;                 // steps of mask entries resident per wave
     constexpr int kMaskWaveBytes = 32 * BN * MaskT<MT>::BYTES;   // 32 rows x 64 keys
     constexpr int kMaskInstr = kMaskWaveBytes / 1024;            // loads per wave and step
@@ -325,7 +329,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         for (int e = 0; e < kMaskInstr; e++) {
             const int rl = (64 / kMaskLPR) * e + lane / kMaskLPR;  // row of the wave's tile
             const int r = min(rl, a.M - 1 - row_first);
-            const int chunk = MADD ? (lane % kMaskLPR) ^ (2 * (rl & 3))
+            const int chunk = MF32 ? (lane % kMaskLPR) ^ (rl & 7)
+                            : MADD ? (lane % kMaskLPR) ^ (2 * (rl & 3))
                                    : (lane & 3) ^ ((lane >> 4) & 3);  // (bits 2-3 of the row number 16 e + lane / 4)
             m_goff[e] = (unsigned)((r * (int)a.ms_m) * MB + 16 * chunk);
             m_goff_last[e] = (unsigned)((r * (int)a.ms_m) * MB + 16 * min(chunk, last_chunk));
@@ -342,6 +347,20 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     };
     // (additive) the lane's entries of 16-key slice tp of a staged step: four words, the entries of score registers
     // 8 (tp & 1) + 0 .. 3 (two words) and + 4 .. 7 (two words) of tile tp >> 1
+    // (fp32 entries) 256 bytes per staged row, sixteen lanes per row, instruction e carries rows 4 e .. 4 e + 3; the
+    // sixteen chunks of a row are XOR-swizzled with bits 0-2 of the row number.  mask_half: the lane's four entries of
+    // half-slice hs = 2 tp + j (score registers 8 (tp & 1) + 4 j .. + 3 of tile tp >> 1): chunk 2 hs + half of its row.
+    auto mask_half = [&](int hs, v4f& e) {
+        const unsigned char* row = smem + F::TOTAL + wave * kMaskWaveBytes + l32 * (BN * MB);
+        e = *reinterpret_cast<const v4f*>(row + ((32 * hs) ^ (16 * ((l32 & 7) ^ half))));
+    };
+    // the same four entries from memory (the path that redoes a step: the staged ones may have been replaced by then)
+    auto mask_half_global = [&](int n_first, int hs, v4f& e) {
+        const int64_t row = min(my_m, a.M - 1);
+        const float* rp = static_cast<const float*>(a.mask) + (int64_t)b * a.ms_b + (int64_t)h * a.ms_h + row * a.ms_m;
+        const int key = min(n_first + 8 * hs + 4 * half, ((a.N - 1) / 4) * 4);  // (keys past kv_len: any readable entry, unused)
+        e = *reinterpret_cast<const v4f*>(rp + key);
+    };
     auto mask_entries = [&](int slot, int tp, unsigned (&w)[4]) {
         const unsigned char* row = smem + F::TOTAL + (slot * kFastWaves + wave) * kMaskWaveBytes + l32 * (BN * MB) + 8 * half;
         const v2u* piece = reinterpret_cast<const v2u*>(row + 32 * (tp ^ (l32 & 3)));
@@ -442,7 +461,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
     constexpr int QK_SLOTS = 2 * F::KSTEPS;
     constexpr int PV_SLOTS = 4 * F::DTILES;
     constexpr int NSLOTS = QK_SLOTS + PV_SLOTS;
-    constexpr int DEFER = (D == 64 && INT8) ? 4 : 0;        // exponential units moved into the MFMA phase (measured per instance)
+    constexpr int DEFER = (D == 64 && INT8 && !MF32) ? 4 : 0;  // exponential units moved into the MFMA phase (measured per instance;
+                                                               // fp32 mask entries: every unit reads them before the slot is refilled)
     constexpr bool kWholeRowSums = QB == 2 && !CAUSAL;      // row sums by the matrix core: every lane holds its whole row's sum
     constexpr int KDIST = 4 < QK_SLOTS ? 4 : QK_SLOTS;      // K fragments in flight
     constexpr int VDIST = 3 < QK_SLOTS ? 3 : QK_SLOTS - 1;  // V fragments in flight
@@ -509,7 +529,32 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         // (a row that sees no key at all, qo_len > kv_len under the causal flag, keeps a finite reference
         // point: its exponentials are then exp2(-inf) = 0 and it ends with l = 0)
         m_i = fmaxf((row_pair_max(raw_max) - BIAS) * sc, -1.0e30f);
-        if (MASK) m_i = -INFINITY;  // no visible key seen yet: the first step with one sets the reference point
+        if (MASK && !MADD) m_i = -INFINITY;  // no visible key seen yet: the first step with one sets the reference point
+        if constexpr (MADD) {  // the maximum of score * scale + entry over the first tile (its entries are staged)
+            float mx = -INFINITY;
+            sfor<4>([&](auto tc) {
+                constexpr int tp = decltype(tc)::value, kt = tp >> 1;
+                float e8[8];
+                if constexpr (MF32) {
+                    v4f lo, hi;
+                    mask_half(2 * tp, lo);
+                    mask_half(2 * tp + 1, hi);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) { e8[c] = lo[c]; e8[4 + c] = hi[c]; }
+                } else {
+                    unsigned w4[4];
+                    mask_entries(0, tp, w4);
+#pragma unroll
+                    for (int c = 0; c < 8; c++) e8[c] = mask_entry<MT>(w4[c >> 1], c & 1);
+                }
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const int bits = sbuf[0][kt][8 * (tp & 1) + c];
+                    mx = fmaxf(mx, __builtin_fmaf(as_f(bits) - BIAS, sc, e8[c]));
+                }
+            });
+            m_i = fmaxf(row_pair_max(mx), -1.0e30f);
+        }
     }
     int mslot = 0;  // slot of the current step's mask bytes (step % 3)
 
@@ -575,22 +620,29 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         const int mslot_next = mslot == kMaskSlots - 1 ? 0 : mslot + 1;
         // (additive: the entries of step + 1, into the slot that step - 1 left; ahead of the K/V loads, because they
         // are the ones waited for first: at the end of the coming matrix phase)
-        if constexpr (MADD) dma_mask(min(step + 1, nsteps - 1), mslot_next);
+        if constexpr (MADD && !MF32) dma_mask(min(step + 1, nsteps - 1), mslot_next);
         sfor<NDMA_KV>([&](auto ec) { dma_unit(ec, IC<HIDES>{}, (step + 3) & 3, k_fetch, k_tile, (step + 2) & 3, v_fetch, v_tile); });
         if constexpr (MASK && !MADD) dma_mask(min(step + 2, nsteps - 1), mslot_next == kMaskSlots - 1 ? 0 : mslot_next + 1);  // the mask bytes of step + 2
         vec16 pf[4];
         float lsum = 0.0f;
         const float sc_e = sc;  // this step's scale (sc moves on to the next step below)
         unsigned mw[2][2] = {{0, 0}, {0, 0}};  // (bool mask) the lane's mask bytes of the 16-key slice in work and of the next one
-        unsigned me[2][4] = {};                // (additive mask) the lane's entries of the slice in work and of the next one
+        unsigned me[2][4] = {};                // (additive 16-bit mask) the lane's entries of the slice in work and of the next one
+        v4f mf[2] = {};                        // (additive fp32 mask) the lane's entries of the half-slice in work and of the next one
         if constexpr (MASK && !MADD) mask_words(mslot, 0, mw[0][0], mw[0][1]);
-        if constexpr (MADD) mask_entries(mslot, 0, me[0]);
+        if constexpr (MADD && !MF32) mask_entries(mslot, 0, me[0]);
+        if constexpr (MF32) mask_half(0, mf[0]);
         auto exp_unit = [&](auto uc) {  // two scores -> two 16-bit P values
             constexpr int u = decltype(uc)::value;
             constexpr int tp = u >> 2, w = u & 3, kt = tp >> 1, i0 = 8 * (tp & 1) + 2 * w;
             const int b0 = sbuf[P][kt][i0], b1 = sbuf[P][kt][i0 + 1];
             float t0 = neg_m, t1 = neg_m;
-            if constexpr (MADD) {  // the mask entry joins the exponent: score * scale + entry - m
+            if constexpr (MF32) {  // the mask entry joins the exponent: score * scale + entry - m
+                constexpr int hs = 2 * tp + (w >> 1);
+                if constexpr ((w & 1) == 0 && hs < 7) mask_half(hs + 1, mf[(hs + 1) & 1]);
+                t0 += mf[hs & 1][2 * (w & 1)];
+                t1 += mf[hs & 1][2 * (w & 1) + 1];
+            } else if constexpr (MADD) {
                 if constexpr (w == 0 && tp < 3) mask_entries(mslot, tp + 1, me[(tp + 1) & 1]);
                 const unsigned word = me[tp & 1][w];
                 t0 += mask_entry<MT>(word, 0);
@@ -627,6 +679,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
             lsum = PVT::dot2_ones(pf[3], 2, lsum);
             lsum = PVT::dot2_ones(pf[3], 3, lsum);
         }
+        // (fp32 mask entries: the last one of this step has been read; the one slot takes those of the next step)
+        if constexpr (MF32) dma_mask(min(step + 1, nsteps - 1), 0);
         // A lane's 32 P of a step sum to less than kSumLimit, or the step is redone: so no P overflows the
         // 16-bit type (nor does a sum or a product with V come near the fp32 range), and a row whose scores
         // rise keeps its reference point within log2(kSumLimit) of its maximum.  Wave-wide decision; rare
@@ -650,14 +704,25 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
                     float past_end = 0.0f;  // number of the lane's keys of this step that lie past kv_len
                     sfor<4>([&](auto tc) {
                         constexpr int tp = decltype(tc)::value, kt = tp >> 1;
-                        unsigned w4[4];
-                        mask_entries(mslot, tp, w4);
+                        float e8[8];
+                        if constexpr (MF32) {
+                            v4f lo, hi;
+                            mask_half_global(n0, 2 * tp, lo);
+                            mask_half_global(n0, 2 * tp + 1, hi);
+#pragma unroll
+                            for (int c = 0; c < 4; c++) { e8[c] = lo[c]; e8[4 + c] = hi[c]; }
+                        } else {
+                            unsigned w4[4];
+                            mask_entries(mslot, tp, w4);
+#pragma unroll
+                            for (int c = 0; c < 8; c++) e8[c] = mask_entry<MT>(w4[c >> 1], c & 1);
+                        }
 #pragma unroll
                         for (int c = 0; c < 8; c++) {
                             const int i = 8 * (tp & 1) + c;
                             const int bits = sbuf[P][kt][i];
                             const float x = as_f(bits);
-                            float sv = __builtin_fmaf(folded ? x - BIAS : x, sc_e, mask_entry<MT>(w4[c >> 1], c & 1));
+                            float sv = __builtin_fmaf(folded ? x - BIAS : x, sc_e, e8[c]);
                             if (x == -INFINITY) {  // past kv_len
                                 sv = -INFINITY;
                                 past_end += 1.0f;
@@ -861,7 +926,8 @@ __global__ __launch_bounds__(kFastThreads, kFastWgPerCu) void sage_attn_fwd_fast
         if (step + 3 < nsteps) { v_fetch += v_tile_bytes; v_tile++; }
         __builtin_amdgcn_s_setprio(0);
         // (additive mask: the entries of the next step, requested ahead of this step's K/V loads, have landed)
-        if constexpr (MADD) __builtin_amdgcn_s_waitcnt(0x0F70 | NDMA_KV);
+        if constexpr (MF32) __builtin_amdgcn_s_waitcnt(0x0F70);
+        else if constexpr (MADD) __builtin_amdgcn_s_waitcnt(0x0F70 | NDMA_KV);
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): every fragment read of this phase has returned
         __builtin_amdgcn_s_barrier();        // phase switch: this wave goes back to the VALU
         __builtin_amdgcn_sched_barrier(0);

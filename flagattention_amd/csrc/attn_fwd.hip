@@ -496,11 +496,12 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
     const bool is_bool = p.mask_kind == SAGE_MASK_BOOL || p.mask_kind == SAGE_MASK_BOOL_PADDED ||
                          p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL;
     a.mask_padded = p.mask_kind == SAGE_MASK_BOOL_PADDED || p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL ||
-                    p.mask_kind == SAGE_MASK_F16_PADDED || p.mask_kind == SAGE_MASK_BF16_PADDED;
+                    p.mask_kind == SAGE_MASK_F16_PADDED || p.mask_kind == SAGE_MASK_BF16_PADDED ||
+                    p.mask_kind == SAGE_MASK_F32_PADDED;
     a.mask_causal = p.mask_kind == SAGE_MASK_BOOL_PADDED_CAUSAL;
     const bool f16 = p.mask_kind == SAGE_MASK_F16 || p.mask_kind == SAGE_MASK_F16_PADDED;
     const bool bf16 = p.mask_kind == SAGE_MASK_BF16 || p.mask_kind == SAGE_MASK_BF16_PADDED;
-    const bool additive = p.mask_kind == SAGE_MASK_F32 || f16 || bf16;
+    const bool additive = p.mask_kind == SAGE_MASK_F32 || p.mask_kind == SAGE_MASK_F32_PADDED || f16 || bf16;
     a.mask_dt = f16 ? SAGE_F16 : bf16 ? SAGE_BF16 : SAGE_F32;
     if (p.mask_kind != SAGE_MASK_NONE && p.mask_stride_n == 1) {
         // runs of four entries are read with one load where they are naturally aligned
@@ -536,7 +537,7 @@ int launch_attn(const sage_attn_params& p, void* workspace, int64_t workspace_by
         return attn::launch_fast(a, (int)p.head_dim, p.v_dtype, p.causal != 0, stream);
     }
     a.mask_additive = additive;
-    if ((is_bool && attn::fast_serves_mask(a, 1)) || (additive && a.mask_dt != SAGE_F32 && attn::fast_serves_mask(a, 2)))
+    if ((is_bool && attn::fast_serves_mask(a, 1)) || (additive && attn::fast_serves_mask(a, dtype_bytes(a.mask_dt))))
         return attn::launch_fast_masked(a, (int)p.head_dim, p.v_dtype, stream);
     if (p.head_dim == 128) {
         return p.v_dtype == SAGE_BF16 ? launch_mode<128, __bf16>(a, mode, stream)

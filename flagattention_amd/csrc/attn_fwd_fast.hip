@@ -36,11 +36,11 @@ int launch_masked(const AttnArgs& a, hipStream_t stream) {
 // A bool mask tensor the pipelined kernel can stage with 16-byte loads: contiguous along the keys, every row start
 // 16-byte aligned, no load that reaches past the end of a row (kv_len a multiple of 16, or rows that the caller
 // padded with zeros to one), no causal flag on top.
-// (esz: bytes per mask entry, 1 for bool masks, 2 for additive fp16 / bf16 ones; fp32 masks are not staged)
+// (esz: bytes per mask entry, 1 for bool masks, 2 / 4 for additive ones)
 bool fast_serves_mask(const AttnArgs& a, int esz) {
     const int per16 = 16 / esz;  // entries per 16-byte load
-    return a.mask != nullptr && !a.causal && (esz == 1 || esz == 2) && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 &&
-           a.ms_b % per16 == 0 && a.ms_h % per16 == 0 && a.ms_m % per16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 25) &&
+    return a.mask != nullptr && !a.causal && a.ms_n == 1 && ((uintptr_t)a.mask % 16) == 0 &&
+           a.ms_b % per16 == 0 && a.ms_h % per16 == 0 && a.ms_m % per16 == 0 && a.ms_m >= 0 && a.ms_m < (1 << 24) &&
            (a.N % per16 == 0 || a.mask_padded);
 }
 

@@ -1,7 +1,7 @@
-// SageAttention forward for gfx950, pipelined kernel under an additive mask tensor stored as fp16 or bf16: the
-// instances of attn_fast_kernel.h that stage 16-bit mask entries (FlagAttention
+// SageAttention forward for gfx950, pipelined kernel under an additive mask tensor stored as fp16, bf16 or fp32: the
+// instances of attn_fast_kernel.h that stage mask entries of those types (FlagAttention
 // src/flag_attn/sage_attention/attn_qk_int8_per_block.py:37-38,49-50: score + mask entry).  A translation unit of
-// its own: eight more instances of the kernel.
+// its own: twelve more instances of the kernel.
 #include "attn_fast_kernel.h"
 
 namespace sage {
@@ -15,11 +15,12 @@ int launch_additive(const AttnArgs& a, hipStream_t stream) {
     b.total_wg = (int)((int64_t)a.total_wg / a.nq * nq2);
     dim3 grid((unsigned)b.total_wg), block(kFastThreads);
     hipLaunchKernelGGL((sage_attn_fwd_fast_kernel<D, VT, true, 1, MT>), grid, block, 0, stream, b, nq2);
-    return check_launch("sage_attn_fwd_fast_kernel (additive 16-bit mask)");
+    return check_launch("sage_attn_fwd_fast_kernel (additive mask)");
 }
 
 template <int D, typename VT>
 int launch_additive_mt(const AttnArgs& a, hipStream_t stream) {
+    if (a.mask_dt == SAGE_F32) return launch_additive<D, VT, float>(a, stream);
     return a.mask_dt == SAGE_BF16 ? launch_additive<D, VT, __bf16>(a, stream) : launch_additive<D, VT, _Float16>(a, stream);
 }
 

@@ -129,7 +129,7 @@ static int check_attn_params(const sage_attn_params* p) {
     if (p->v_dtype != SAGE_F16 && p->v_dtype != SAGE_BF16)
         return fail(SAGE_E_UNSUPPORTED, "sage_attn_fwd: V must be fp16 or bf16");
     if (!float_dtype_ok(p->out_dtype)) return fail(SAGE_E_INVALID, "sage_attn_fwd: bad out_dtype %d", p->out_dtype);
-    if (p->mask_kind < SAGE_MASK_NONE || p->mask_kind > SAGE_MASK_BF16_PADDED)
+    if (p->mask_kind < SAGE_MASK_NONE || p->mask_kind > SAGE_MASK_F32_PADDED)
         return fail(SAGE_E_INVALID, "sage_attn_fwd: bad mask_kind %d", p->mask_kind);
     if (p->mask_kind != SAGE_MASK_NONE && !p->mask) return fail(SAGE_E_INVALID, "sage_attn_fwd: null mask");
     // 16-byte vector loads: row starts of Q/K (int8) and V (16-bit) must be 16-byte aligned

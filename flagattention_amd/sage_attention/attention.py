@@ -78,19 +78,21 @@ def stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=None):
 
 
 def _additive_mask_is_direct(m: torch.Tensor, kv_len: int) -> bool:
-    """Can the pipelined kernel stage this (already expanded) fp16 / bf16 additive mask as it is?  16-byte loads
-    along the keys: unit stride, 16-byte aligned rows, and no load that passes the end of a row."""
-    return (m.stride(-1) == 1 and m.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in m.stride()[:-1])
-            and m.stride(2) < (1 << 25) and kv_len % 8 == 0)
+    """Can the pipelined kernel stage this (already expanded) fp16 / bf16 / fp32 additive mask as it is?  16-byte
+    loads along the keys: unit stride, 16-byte aligned rows, and no load that passes the end of a row."""
+    per16 = 16 // m.element_size()
+    return (m.stride(-1) == 1 and m.data_ptr() % 16 == 0 and all(s % per16 == 0 for s in m.stride()[:-1])
+            and m.stride(2) < (1 << 24) and kv_len % per16 == 0)
 
 
 def _stage_additive_mask(mask, b, h, qo_len, kv_len):
-    """A copy of an fp16 / bf16 additive mask with unit stride along the keys and rows padded (with zeros) to a
-    multiple of 8 entries, broadcast dimensions kept; None when the copy would pass ``_STAGED_MASK_MAX_BYTES``."""
-    padded = (kv_len + 7) // 8 * 8
+    """A copy of an fp16 / bf16 / fp32 additive mask with unit stride along the keys and rows padded (with zeros) to
+    a multiple of 16 bytes, broadcast dimensions kept; None when the copy would pass ``_STAGED_MASK_MAX_BYTES``."""
+    per16 = 16 // mask.element_size()
+    padded = (kv_len + per16 - 1) // per16 * per16
     m4 = mask.reshape((1,) * (4 - mask.dim()) + tuple(mask.shape))
     bb, hh, mm = m4.shape[0], m4.shape[1], m4.shape[2]
-    if bb * hh * mm * padded * 2 > _STAGED_MASK_MAX_BYTES:
+    if bb * hh * mm * padded * mask.element_size() > _STAGED_MASK_MAX_BYTES:
         return None
     buf = torch.zeros((bb, hh, mm, padded), dtype=mask.dtype, device=mask.device)
     live = buf[..., :kv_len]
@@ -235,19 +237,19 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
                 m = attn_mask
                 if m.dtype == torch.bool:
                     mask_kind = _lib.MASK_BOOL
-                elif m.dtype in (torch.float16, torch.bfloat16):
-                    mask_kind = _lib.MASK_F16 if m.dtype == torch.float16 else _lib.MASK_BF16
-                    # 16-bit additive masks run on the pipelined kernel (no causal flag on top); one whose rows it
-                    # cannot load 16 bytes at a time goes there through a padded copy
+                else:
+                    if m.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+                        m = m.float()  # (float64 or integer masks: the kernel adds fp32 values)
+                    plain, padded_kind = {torch.float16: (_lib.MASK_F16, _lib.MASK_F16_PADDED),
+                                          torch.bfloat16: (_lib.MASK_BF16, _lib.MASK_BF16_PADDED),
+                                          torch.float32: (_lib.MASK_F32, _lib.MASK_F32_PADDED)}[m.dtype]
+                    mask_kind = plain
+                    # additive masks run on the pipelined kernel (no causal flag on top); one whose rows it cannot load
+                    # 16 bytes at a time goes there through a padded copy
                     if not causal and not _additive_mask_is_direct(m.expand(b, h_qo, qo_len, kv_len), kv_len):
                         padded = _staged_additive_cached(m, b, h_qo, qo_len, kv_len, dev)
                         if padded is not None:
-                            m = padded
-                            mask_kind = _lib.MASK_F16_PADDED if m.dtype == torch.float16 else _lib.MASK_BF16_PADDED
-                else:
-                    mask_kind = _lib.MASK_F32
-                    if m.dtype != torch.float32:  # (float64 or integer masks: the kernel adds fp32 values)
-                        m = m.float()
+                            m, mask_kind = padded, padded_kind
                 m = m.expand(b, h_qo, qo_len, kv_len)
         if m is not None and mask_kind == _lib.MASK_NONE:  # a staged mask
             causal_flag = 0

@@ -25,7 +25,7 @@ extern "C" {
 enum sage_dtype { SAGE_F16 = 0, SAGE_BF16 = 1, SAGE_F32 = 2 };
 enum sage_mask_kind { SAGE_MASK_NONE = 0, SAGE_MASK_BOOL = 1, SAGE_MASK_F32 = 2, SAGE_MASK_F16 = 3, SAGE_MASK_BF16 = 4,
                       SAGE_MASK_BOOL_PADDED = 5, SAGE_MASK_BOOL_PADDED_CAUSAL = 6, SAGE_MASK_F16_PADDED = 7,
-                      SAGE_MASK_BF16_PADDED = 8 };
+                      SAGE_MASK_BF16_PADDED = 8, SAGE_MASK_F32_PADDED = 9 };
 enum sage_status {
     SAGE_OK = 0,
     SAGE_E_INVALID = -1,     /* bad argument (shape, dtype, stride, null pointer) */
@@ -84,12 +84,12 @@ int sage_per_block_int8(const sage_quant_params* p, void* stream);
  *                SAGE_MASK_BOOL_PADDED_CAUSAL: a padded mask of which the caller also guarantees mask[m, n] = 0 for
  *                n > m + (kv_len - qo_len) (the causal mask is folded in): the pipelined kernel then does not visit
  *                the key tiles beyond that limit, which the reference would skip one by one as all-False tiles;
- *                SAGE_MASK_F32 / SAGE_MASK_F16 / SAGE_MASK_BF16: additive, in that storage type (:38,50); fp16 / bf16
- *                masks with unit stride along the keys, 16-byte aligned rows and kv_len % 8 == 0 (and no causal flag)
- *                run on the pipelined kernel, every other additive mask on the general one;
- *                SAGE_MASK_F16_PADDED / SAGE_MASK_BF16_PADDED: the same, and the caller guarantees that every mask row
- *                can be read up to the next multiple of 16 bytes past kv_len (any finite values there): such a mask
- *                runs on the pipelined kernel for any kv_len
+ *                SAGE_MASK_F32 / SAGE_MASK_F16 / SAGE_MASK_BF16: additive, in that storage type (:38,50); masks with
+ *                unit stride along the keys, 16-byte aligned rows and kv_len * entry size a multiple of 16 bytes (and
+ *                no causal flag) run on the pipelined kernel, every other additive mask on the general one;
+ *                SAGE_MASK_F16_PADDED / SAGE_MASK_BF16_PADDED / SAGE_MASK_F32_PADDED: the same, and the caller
+ *                guarantees that every mask row can be read up to the next multiple of 16 bytes past kv_len (any finite
+ *                values there): such a mask runs on the pipelined kernel for any kv_len
  *   causal       non-zero adds the bottom-right aligned causal mask n <= m + (N - M), handled
  *                like a bool mask (tiles that are entirely masked are skipped)
  * head_dim must be 64 or 128; heads_q must be a multiple of heads_kv.

@@ -365,14 +365,14 @@ def test_bool_mask_kinds_through_the_c_abi(n, gpu_device):
         _check_masked(o, lse, expected, expected_lse, f"kind {kind}")
         outs.append(o)
     torch.testing.assert_close(outs[0], outs[1], atol=5e-3, rtol=1e-2)
-    p.mask_kind = 9
+    p.mask_kind = 10
     assert lib.sage_attn_fwd(ctypes.byref(p), None) == -1 and b"mask_kind" in lib.sage_hip_last_error()
 
 
 def _additive_case(kind, b, h, m, n, seed, dtype):
     """Additive masks (already in their 16-bit storage type; the oracle adds their fp32 images)."""
     g = torch.Generator().manual_seed(seed)
-    far = -1.0e6 if dtype == torch.bfloat16 else -6.0e4  # (fp16 ends at 65504: -1e6 would be stored as -inf)
+    far = -6.0e4 if dtype == torch.float16 else -1.0e6  # (fp16 ends at 65504: -1e6 would be stored as -inf)
     if kind == "bias":  # a relative-position style bias, per (batch, head)
         mask = torch.randn(b, h, m, n, generator=g) * 3.0
     elif kind == "broadcast":
@@ -399,11 +399,13 @@ def _additive_case(kind, b, h, m, n, seed, dtype):
 
 @pytest.mark.parametrize("kind", ["bias", "broadcast", "key_padding", "blocks", "jumps"])
 @pytest.mark.parametrize("d,vdtype,mdtype", [(128, torch.bfloat16, torch.bfloat16), (128, torch.bfloat16, torch.float16),
-                                             (64, torch.float16, torch.float16), (64, torch.float16, torch.bfloat16)])
-@pytest.mark.parametrize("m,n", [(300, 512), (129, 80), (600, 1040), (200, 257), (64, 64), (700, 333)])
-def test_additive_16bit_masks_on_the_pipelined_kernel(kind, d, vdtype, mdtype, m, n, gpu_device):
-    """fp16 / bf16 additive masks take the pipelined kernel (as they are when their rows can be loaded 16 bytes at a
-    time, through a padded copy otherwise): score + entry as in attn_qk_int8_per_block.py:37-38,49-50, keys past
+                                             (64, torch.float16, torch.float16), (64, torch.float16, torch.bfloat16),
+                                             (128, torch.bfloat16, torch.float32), (64, torch.float16, torch.float32),
+                                             (128, torch.float16, torch.float32)])
+@pytest.mark.parametrize("m,n", [(300, 512), (129, 80), (600, 1040), (200, 257), (64, 64), (700, 333), (40, 1283)])
+def test_additive_masks_on_the_pipelined_kernel(kind, d, vdtype, mdtype, m, n, gpu_device):
+    """fp16 / bf16 / fp32 additive masks take the pipelined kernel (as they are when their rows can be loaded 16 bytes
+    at a time, through a padded copy otherwise): score + entry as in attn_qk_int8_per_block.py:37-38,49-50, keys past
     kv_len at -1e6, no tile skipped.  Against the oracle's tile arithmetic on the fp32 images of the entries."""
     b, hq, hkv = 2, 4, 2
     q8, qs, k8, ks, v = _quantized(52, b, hq, hkv, m, n, d, vdtype)
@@ -417,14 +419,15 @@ def test_additive_16bit_masks_on_the_pipelined_kernel(kind, d, vdtype, mdtype, m
     torch.testing.assert_close(lse.cpu()[~normal], expected_lse[~normal], atol=1.0, rtol=1e-5)
 
 
-def test_additive_16bit_mask_views_and_the_general_kernel_agree(gpu_device):
-    """The same bf16 additive mask as a contiguous tensor (pipelined kernel as it is), as a column slice of a wider
+@pytest.mark.parametrize("mdtype", [torch.bfloat16, torch.float32])
+def test_additive_mask_views_and_the_general_kernel_agree(mdtype, gpu_device):
+    """The same additive mask as a contiguous tensor (pipelined kernel as it is), as a column slice of a wider
     tensor (padded copy), and with a causal flag on top (general kernel: a causal flag is not folded into an additive
     mask): the first two give the same bits, the third matches the oracle's mask + causal arithmetic."""
     b, hq, hkv, m, n = 1, 2, 2, 260, 328
     q8, qs, k8, ks, v = _quantized(53, b, hq, hkv, m, n, 128, torch.bfloat16)
     g = torch.Generator().manual_seed(29)
-    wide = (torch.randn(b, hq, m, n + 24, generator=g) * 2.0).to(torch.bfloat16).to(gpu_device)
+    wide = (torch.randn(b, hq, m, n + 24, generator=g) * 2.0).to(mdtype).to(gpu_device)
     view = wide[..., 3:3 + n]
     o1, lse1 = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=view.contiguous(), return_lse=True, output_dtype=torch.float32)
     o2, lse2 = _run(gpu_device, q8, qs, k8, ks, v, attn_mask=view, return_lse=True, output_dtype=torch.float32)
