@@ -277,8 +277,9 @@ def main():
     ap.add_argument("--op", default="sage_attention", choices=["sage_attention", "flash_attention"],
                     help="sage_attention (default): K mean + quantization + INT8-QK forward; flash_attention: the dense 16-bit forward")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mask", default="none", choices=["none", "bool"],
-                    help="side path of --op sage_attention: forward under a seeded [1, 1, M, N] bool mask (30 %% hidden)")
+    ap.add_argument("--mask", default="none", choices=["none", "bool", "bf16", "fp16", "fp32"],
+                    help="side path of --op sage_attention: forward under a seeded [1, 1, M, N] mask: bool (30 %% hidden) or "
+                         "additive N(0, 1) entries stored as bf16 / fp16 / fp32")
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="side path of --op flash_attention: dropout probability of the forward call")
     ap.add_argument("--min-warmup-seconds", type=float, default=0.15,
@@ -312,6 +313,10 @@ def main():
     if args.mask == "bool":
         mask_cpu = torch.rand(1, 1, n, n, generator=torch.Generator().manual_seed(43)) > 0.3
         mask_dev = mask_cpu.to(dev)
+    elif args.mask != "none":
+        mdt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.mask]
+        mask_dev = torch.randn(1, 1, n, n, generator=torch.Generator().manual_seed(43)).to(mdt).to(dev)
+        mask_cpu = mask_dev.cpu().float()  # (the oracle adds the fp32 images of the stored entries)
 
     def step(ev=None):
         if ev:
@@ -416,9 +421,10 @@ def main():
         "dtype": "int8 QK^T (int32 acc) + bf16 PV (fp32 acc), fp32 softmax" if dtype == torch.bfloat16
         else "int8 QK^T (int32 acc) + fp16 PV (fp32 acc), fp32 softmax",
         "data": "synthetic (seed 42, N(0,1) generated on CPU, copied to HBM before timing)",
-        "config": {"workload": desc + ("_boolmask" if mask_dev is not None else ""), "batch": b, "heads": h, "seq_len": n,
+        "config": {"workload": desc + ("" if mask_dev is None else "_boolmask" if args.mask == "bool" else "_additive_%s_mask" % args.mask), "batch": b, "heads": h, "seq_len": n,
                    "head_dim": d, "layout": layout, "causal": causal, "smooth_k": smooth, "blkq": 128, "blkk": 64,
-                   "attn_mask": "[1, 1, M, N] bool, 30 % hidden, seed 43" if mask_dev is not None else None},
+                   "attn_mask": None if mask_dev is None else "[1, 1, M, N] bool, 30 % hidden, seed 43" if args.mask == "bool"
+                   else "[1, 1, M, N] additive N(0, 1) entries stored as %s, seed 43" % args.mask},
         "pct_of_mixed_mfma_peak": round(100 * value / PEAK_MIXED_TOPS, 2),
         "attention_only": {
             "us_per_call_avg": round(attn_avg * 1e3, 1),

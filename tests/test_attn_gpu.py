@@ -811,3 +811,24 @@ def test_additive_masks_of_other_float_types(mask_dtype, m, n, gpu_device):
     expected, expected_lse = O.attention_dequant(q8, k8, v, qs, ks, attn_mask=mask.float())
     _gate(o, expected)
     torch.testing.assert_close(lse.cpu(), expected_lse, atol=6e-3, rtol=1e-4)
+
+
+def test_torch_library_operators_under_torch_compile(gpu_device):
+    """A function that calls torch.ops.flagattention_amd.* traced by torch.compile (aot_eager: no code generator
+    needed) gives the bits of the plain Python calls."""
+    import flagattention_amd.torch_ops  # noqa: F401
+    from flag_attn import sage_attention as sa
+
+    ops = torch.ops.flagattention_amd
+    g = torch.Generator().manual_seed(77)
+    q, k, v = (torch.randn(1, 2, 200, 64, generator=g).half().to(gpu_device) for _ in range(3))
+
+    def attn(q, k, v):
+        q8, qs, k8, ks = ops.per_block_int8(q, k, smooth_k=True)
+        o, lse = ops.sage_attention_forward(q8, k8, v, qs, ks, "HND", None, torch.float16, True, True)
+        return o * 2.0, lse
+
+    o_c, lse_c = torch.compile(attn, backend="aot_eager", fullgraph=True)(q, k, v)
+    q8, qs, k8, ks = sa.per_block_int8(q, k, smooth_k=True)
+    o_e, lse_e = sa.forward(q8, k8, v, qs, ks, return_lse=True, causal=True)
+    assert torch.equal(o_c, o_e * 2.0) and torch.equal(lse_c, lse_e)

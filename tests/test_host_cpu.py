@@ -321,3 +321,26 @@ def test_only_the_lds_load_sequence_touches_m0(tmp_path):
         assert not other, other[:5]
         loads = sum(1 for ln in out.read_text().splitlines() if ln.strip().startswith("global_load_lds_dwordx4"))
         assert loads == len(mentions)
+
+
+def test_torch_library_operators_have_shape_functions():
+    """torch.ops.flagattention_amd.*: registered, and their shape functions (run here on fake GPU tensors, no GPU
+    needed) give the shapes, dtypes and devices of the real calls, the empty fp32 CPU lse of return_lse=False
+    included."""
+    import torch
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    import flagattention_amd.torch_ops  # noqa: F401  (registers the operators)
+
+    ops = torch.ops.flagattention_amd
+    with FakeTensorMode():
+        q = torch.empty(2, 300, 4, 64, dtype=torch.float16, device="cuda")  # NHD
+        k = torch.empty(2, 500, 2, 64, dtype=torch.float16, device="cuda")
+        q8, qs, k8, ks = ops.per_block_int8(q, k, tensor_layout="NHD", smooth_k=True)
+        assert q8.shape == q.shape and k8.shape == k.shape and q8.dtype == k8.dtype == torch.int8
+        assert tuple(qs.shape) == (2, 4, 3) and tuple(ks.shape) == (2, 2, 8) and qs.dtype == ks.dtype == torch.float32
+        o, lse = ops.sage_attention_forward(q8, k8, k, qs, ks, "NHD", None, torch.bfloat16, True, True)
+        assert o.shape == q.shape and o.dtype == torch.bfloat16 and o.device.type == "cuda"
+        assert tuple(lse.shape) == (2, 4, 300) and lse.dtype == torch.float32
+        o, lse = ops.sage_attention_forward(q8, k8, k, qs, ks, "NHD")
+        assert o.dtype == torch.float16 and tuple(lse.shape) == (0,) and lse.device.type == "cpu"
