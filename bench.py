@@ -129,6 +129,13 @@ WORKLOADS = {
 }
 
 
+DATA_NOTE = {
+    "c1": "N(0,1)", "c2": "N(0,1)", "c5": "N(0,1)",
+    "c3": "N(0,1), K plus a per-(head, channel) offset of N(0, 4)",
+    "c4": "N(0,1) with 1 % of the (head, channel) pairs of Q and K scaled by 20, V uniform in (-1, 1)",
+}
+
+
 def make_inputs(name, device):
     b, h, n, d, dtype, layout, causal, _ = WORKLOADS[name]
     g = torch.Generator().manual_seed(42)
@@ -420,7 +427,7 @@ def main():
         "vs_baseline": None,
         "dtype": "int8 QK^T (int32 acc) + bf16 PV (fp32 acc), fp32 softmax" if dtype == torch.bfloat16
         else "int8 QK^T (int32 acc) + fp16 PV (fp32 acc), fp32 softmax",
-        "data": "synthetic (seed 42, N(0,1) generated on CPU, copied to HBM before timing)",
+        "data": "synthetic (seed 42, %s, generated on CPU, copied to HBM before timing)" % DATA_NOTE[name],
         "config": {"workload": desc + ("" if mask_dev is None else "_boolmask" if args.mask == "bool" else "_additive_%s_mask" % args.mask), "batch": b, "heads": h, "seq_len": n,
                    "head_dim": d, "layout": layout, "causal": causal, "smooth_k": smooth, "blkq": 128, "blkk": 64,
                    "attn_mask": None if mask_dev is None else "[1, 1, M, N] bool, 30 % hidden, seed 43" if args.mask == "bool"

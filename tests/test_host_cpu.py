@@ -310,7 +310,7 @@ def test_only_the_lds_load_sequence_touches_m0(tmp_path):
     import subprocess
 
     csrc = os.path.join(ROOT, "flagattention_amd", "csrc")
-    for unit in ("attn_fwd_fast.hip", "flash_fwd.hip"):
+    for unit in ("attn_fwd_fast.hip", "attn_fwd_fast_addmask.hip", "flash_fwd.hip"):
         out = tmp_path / (unit + ".s")
         subprocess.run(["/opt/rocm/bin/hipcc", "-O3", "-std=c++17", "--offload-arch=gfx950", "-ffp-contract=off", "-Xclang",
                         "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", "-o", str(out),
