@@ -53,7 +53,9 @@ def stage_bool_mask(mask, b, h, qo_len, kv_len, causal, device=None):
 
     ``forward`` stages on its own and keeps the last staged mask of a device (found again through the source
     mask's storage address, version counter, shape and strides); a caller that reuses one mask over many calls
-    (all layers of a model) can stage it once here and pass the result as ``attn_mask``."""
+    (all layers of a model) can stage it once here and pass the result as ``attn_mask``.  The copy is enqueued on
+    the current stream, like any torch operation: a call on another stream has to be ordered behind it by the
+    caller."""
     padded = (kv_len + 15) // 16 * 16
     if mask is None:
         bb, hh, mm = 1, 1, qo_len
@@ -100,8 +102,9 @@ def _stage_additive_mask(mask, b, h, qo_len, kv_len):
     return live.expand(b, h, qo_len, kv_len)
 
 
-def _staged_additive_cached(mask, b, h, qo_len, kv_len, device):
-    key = ("additive", mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, b, h, qo_len, kv_len)
+def _staged_additive_cached(mask, b, h, qo_len, kv_len, device, stream):
+    key = ("additive", mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, b, h, qo_len, kv_len,
+           stream)
     hit = _STAGED.get(device.index)
     if hit is not None and hit[0] == key:
         return hit[1]
@@ -111,13 +114,15 @@ def _staged_additive_cached(mask, b, h, qo_len, kv_len, device):
     return staged
 
 
-def _staged_cached(mask, b, h, qo_len, kv_len, causal, device):
+def _staged_cached(mask, b, h, qo_len, kv_len, causal, device, stream):
     """``stage_bool_mask`` behind a one-entry cache per device: the same mask object contents (storage address,
-    version counter: every in-place write bumps it) under the same call shape is not staged again."""
+    version counter: every in-place write bumps it) under the same call shape is not staged again.  The stream is
+    part of the key: the copy was enqueued on the stream that was current then, and only launches on that stream
+    are ordered behind it."""
     if mask is None:
-        key = (None, b, h, qo_len, kv_len, causal)
+        key = (None, b, h, qo_len, kv_len, causal, stream)
     else:
-        key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), b, h, qo_len, kv_len, causal)
+        key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), b, h, qo_len, kv_len, causal, stream)
     hit = _STAGED.get(device.index)
     if hit is not None and hit[0] == key:
         return hit[1]
@@ -209,6 +214,7 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
                 lse.fill_(float("-inf"))
             return o, lse
 
+        stream = current_stream_ptr(dev)
         # ---- the mask as the library takes it
         mask_kind, causal_flag, m = _lib.MASK_NONE, 1 if causal else 0, None
         if isinstance(attn_mask, StagedBoolMask):
@@ -226,11 +232,11 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
                 # bool masks run on the pipelined kernel; one that it cannot stage as it is (rows that are not 16-byte
                 # aligned, kv_len not a multiple of 16, a causal flag on top) goes there through a padded copy
                 if causal or not _bool_mask_is_direct(attn_mask.expand(b, h_qo, qo_len, kv_len), kv_len):
-                    staged = _staged_cached(attn_mask, b, h_qo, qo_len, kv_len, causal, dev)
+                    staged = _staged_cached(attn_mask, b, h_qo, qo_len, kv_len, causal, dev, stream)
             elif attn_mask is None and causal and qo_len > kv_len:
                 # rows that see no key follow the reference's mask arithmetic (-1e6, whole-tile skip), which the
                 # pipelined kernel implements for mask tensors: hand it the causal mask as one
-                staged = _staged_cached(None, b, h_qo, qo_len, kv_len, True, dev)
+                staged = _staged_cached(None, b, h_qo, qo_len, kv_len, True, dev, stream)
             if staged is not None:
                 m = staged.tensor
             elif attn_mask is not None:
@@ -247,7 +253,7 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
                     # additive masks run on the pipelined kernel (no causal flag on top); one whose rows it cannot load
                     # 16 bytes at a time goes there through a padded copy
                     if not causal and not _additive_mask_is_direct(m.expand(b, h_qo, qo_len, kv_len), kv_len):
-                        padded = _staged_additive_cached(m, b, h_qo, qo_len, kv_len, dev)
+                        padded = _staged_additive_cached(m, b, h_qo, qo_len, kv_len, dev, stream)
                         if padded is not None:
                             m, mask_kind = padded, padded_kind
                 m = m.expand(b, h_qo, qo_len, kv_len)
@@ -281,7 +287,6 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None,
         p.q_scale, p.k_scale = q_scale.data_ptr(), k_scale.data_ptr()
         p.lse = lse.data_ptr() if return_lse else None
         p.mask = None if m is None else m.data_ptr()
-        stream = current_stream_ptr(dev)
         if ws_bytes > 0:
             ws = split_workspace(dev, stream, ws_bytes)
             _lib.check(lib.sage_attn_fwd_ws(p_ref, ws.data_ptr(), ws.numel(), stream), "sage_attn_fwd_ws")

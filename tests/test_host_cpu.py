@@ -174,7 +174,7 @@ def test_bool_mask_staging_copy():
 
 def test_staged_mask_cache_key_and_cap(monkeypatch):
     """The one-entry cache behind forward's staging: the same mask under the same call shape is staged once; an
-    in-place write (version counter), another shape or another causal flag stages again; the source mask is kept
+    in-place write (version counter), another shape, another causal flag or another stream stages again; the source mask is kept
     alive with the entry, so its address cannot come back as another tensor.  Copies above the cap are refused."""
     import torch
 
@@ -183,15 +183,18 @@ def test_staged_mask_cache_key_and_cap(monkeypatch):
     dev = torch.device("cpu")
     A._STAGED.clear()
     mask = torch.rand((1, 1, 9, 37)) > 0.5
-    s1 = A._staged_cached(mask, 2, 3, 9, 37, False, dev)
-    assert A._staged_cached(mask, 2, 3, 9, 37, False, dev) is s1
-    assert A._staged_cached(mask.view(1, 1, 9, 37), 2, 3, 9, 37, False, dev) is s1  # another view of the same data
+    s1 = A._staged_cached(mask, 2, 3, 9, 37, False, dev, 0)
+    assert A._staged_cached(mask, 2, 3, 9, 37, False, dev, 0) is s1
+    assert A._staged_cached(mask.view(1, 1, 9, 37), 2, 3, 9, 37, False, dev, 0) is s1  # another view of the same data
     assert A._STAGED[None][2] is mask
     mask[0, 0, 0, 0] = not bool(mask[0, 0, 0, 0])  # in-place write: staged again, with the new value
-    s2 = A._staged_cached(mask, 2, 3, 9, 37, False, dev)
+    s2 = A._staged_cached(mask, 2, 3, 9, 37, False, dev, 0)
     assert s2 is not s1 and torch.equal(s2.tensor, mask.expand(2, 3, 9, 37))
-    assert A._staged_cached(mask, 2, 3, 9, 37, True, dev) is not s2
-    assert A._staged_cached(None, 1, 2, 12, 7, True, dev) is A._staged_cached(None, 1, 2, 12, 7, True, dev)
+    assert A._staged_cached(mask, 2, 3, 9, 37, True, dev, 0) is not s2
+    assert A._staged_cached(None, 1, 2, 12, 7, True, dev, 0) is A._staged_cached(None, 1, 2, 12, 7, True, dev, 0)
+    # another stream: the copy of the first one is not ordered before launches on this one
+    s3 = A._staged_cached(mask, 2, 3, 9, 37, False, dev, 0)
+    assert A._staged_cached(mask, 2, 3, 9, 37, False, dev, 12345) is not s3
     monkeypatch.setattr(A, "_STAGED_MASK_MAX_BYTES", 1024)
     assert A.stage_bool_mask(torch.ones((2, 3, 9, 37), dtype=torch.bool), 2, 3, 9, 37, False) is None
     assert A.stage_bool_mask(torch.ones((1, 1, 9, 37), dtype=torch.bool), 2, 3, 9, 37, False) is not None
